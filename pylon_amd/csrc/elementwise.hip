@@ -1,0 +1,184 @@
+// Row-wise kernels of the decoder: embedding gather, RMSNorm (alone, or fused with the
+// residual sum that precedes it), and the gated activation of the feed-forward.
+// All reductions and all arithmetic are in float; only loads and stores see bf16.
+#include "common.h"
+
+// ---- embedding ------------------------------------------------------------------
+// out[t, :] = table[ids[t], :] * scale, written as float (the residual stream).
+template <typename T>
+__global__ void embed_kernel(float* __restrict__ out, const T* __restrict__ table,
+                             const int* __restrict__ ids, int hidden, int vocab, float scale) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  // The host checks ids; the clamp only keeps a bad id from reading outside the table.
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const T* row = table + static_cast<size_t>(id) * hidden;
+  float* dst = out + static_cast<size_t>(t) * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(row[i]) * scale;
+}
+
+extern "C" int pylon_embed(float* out, const void* table, int table_dtype, const int* ids,
+                           int tokens, int hidden, int vocab, float scale, hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(table_dtype), "embed: unknown table dtype %d", table_dtype);
+  PYLON_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "embed: bad sizes tokens=%d hidden=%d vocab=%d",
+                tokens, hidden, vocab);
+  if (tokens == 0) return 0;
+  dim3 grid(tokens), block(256);
+  if (table_dtype == PYLON_F32)
+    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, out, (const float*)table, ids,
+                       hidden, vocab, scale);
+  else
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, out, (const bf16_t*)table, ids,
+                       hidden, vocab, scale);
+  PYLON_LAUNCHED("embed");
+}
+
+// ---- RMSNorm ----------------------------------------------------------------------
+// y = (x * 1/sqrt(mean(x^2) + eps)) * w, in float, rounded once on the store.
+// One workgroup per output row. `row_idx` (optional) picks the input row of each
+// output row. With `delta`, the input is resid + delta (float sum); `write_resid`
+// stores that sum back into resid (only meaningful without row_idx).
+template <typename TX, typename TD, typename TO>
+__global__ void rmsnorm_kernel(TO* __restrict__ out, TX* x, const TD* __restrict__ delta,
+                               const float* __restrict__ w, const int* __restrict__ row_idx,
+                               int dim, float eps, int write_resid) {
+  __shared__ float scratch[16];
+  const int r_out = blockIdx.x;
+  const int r_in = row_idx ? row_idx[r_out] : r_out;
+  TX* xr = x + static_cast<size_t>(r_in) * dim;
+  const TD* dr = delta ? delta + static_cast<size_t>(r_in) * dim : nullptr;
+  TO* yr = out + static_cast<size_t>(r_out) * dim;
+
+  constexpr int KEEP = 8;  // elements per thread held in registers
+  float held[KEEP];
+  float ss = 0.f;
+  int n = 0;
+  for (int i = threadIdx.x; i < dim; i += blockDim.x, ++n) {
+    float v = to_float(xr[i]);
+    if (dr) {
+      v += to_float(dr[i]);
+      if (write_resid) xr[i] = from_float<TX>(v);
+    }
+    if (n < KEEP) held[n] = v;
+    ss += v * v;
+  }
+  const float total = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(total / static_cast<float>(dim) + eps);
+  n = 0;
+  for (int i = threadIdx.x; i < dim; i += blockDim.x, ++n) {
+    float v;
+    if (n < KEEP) {
+      v = held[n];
+    } else {
+      v = to_float(xr[i]);
+      if (dr && !write_resid) v += to_float(dr[i]);
+    }
+    yr[i] = from_float<TO>((v * inv) * w[i]);
+  }
+}
+
+template <typename TX, typename TD>
+static void launch_rmsnorm_out(void* out, int out_dtype, TX* x, const TD* delta, const float* w,
+                               const int* row_idx, int rows, int dim, float eps, int write_resid,
+                               hipStream_t stream) {
+  dim3 grid(rows), block(256);
+  if (out_dtype == PYLON_F32)
+    hipLaunchKernelGGL((rmsnorm_kernel<TX, TD, float>), grid, block, 0, stream, (float*)out, x, delta,
+                       w, row_idx, dim, eps, write_resid);
+  else
+    hipLaunchKernelGGL((rmsnorm_kernel<TX, TD, bf16_t>), grid, block, 0, stream, (bf16_t*)out, x,
+                       delta, w, row_idx, dim, eps, write_resid);
+}
+
+// out[r] = rmsnorm(x[idx(r)]) for any input dtype.
+extern "C" int pylon_rmsnorm(void* out, int out_dtype, const void* x, int x_dtype, const float* w,
+                             const int* row_idx, int rows, int dim, float eps, hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(out_dtype) && pylon_valid_dtype(x_dtype), "rmsnorm: unknown dtype");
+  PYLON_REQUIRE(rows >= 0 && dim > 0, "rmsnorm: bad sizes rows=%d dim=%d", rows, dim);
+  PYLON_REQUIRE(eps >= 0.f, "rmsnorm: eps must not be negative");
+  if (rows == 0) return 0;
+  if (x_dtype == PYLON_F32)
+    launch_rmsnorm_out<float, float>(out, out_dtype, (float*)x, nullptr, w, row_idx, rows, dim, eps, 0,
+                                     stream);
+  else
+    launch_rmsnorm_out<bf16_t, bf16_t>(out, out_dtype, (bf16_t*)x, nullptr, w, row_idx, rows, dim, eps,
+                                       0, stream);
+  PYLON_LAUNCHED("rmsnorm");
+}
+
+// resid (float) += delta, then out = rmsnorm(resid). With row_idx the sum is formed only
+// for the picked rows and resid is left untouched.
+extern "C" int pylon_add_rmsnorm(void* out, int out_dtype, float* resid, const void* delta,
+                                 int delta_dtype, const float* w, const int* row_idx, int rows,
+                                 int dim, float eps, hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(out_dtype), "add_rmsnorm: unknown out dtype");
+  PYLON_REQUIRE(delta == nullptr || pylon_valid_dtype(delta_dtype), "add_rmsnorm: unknown delta dtype");
+  PYLON_REQUIRE(rows >= 0 && dim > 0, "add_rmsnorm: bad sizes rows=%d dim=%d", rows, dim);
+  if (rows == 0) return 0;
+  const int write_resid = (delta != nullptr && row_idx == nullptr) ? 1 : 0;
+  if (delta == nullptr || delta_dtype == PYLON_F32)
+    launch_rmsnorm_out<float, float>(out, out_dtype, resid, (const float*)delta, w, row_idx, rows, dim,
+                                     eps, write_resid, stream);
+  else
+    launch_rmsnorm_out<float, bf16_t>(out, out_dtype, resid, (const bf16_t*)delta, w, row_idx, rows,
+                                      dim, eps, write_resid, stream);
+  PYLON_LAUNCHED("add_rmsnorm");
+}
+
+// resid (float) += delta, nothing else (the last residual sum when no norm follows).
+template <typename TD>
+__global__ void add_kernel(float* __restrict__ resid, const TD* __restrict__ delta, size_t n) {
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (; i < n; i += step) resid[i] += to_float(delta[i]);
+}
+
+extern "C" int pylon_residual_add(float* resid, const void* delta, int delta_dtype, long long count,
+                                  hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(delta_dtype), "residual_add: unknown dtype");
+  PYLON_REQUIRE(count >= 0, "residual_add: negative count");
+  if (count == 0) return 0;
+  long long blocks = (count + 255) / 256;
+  if (blocks > 65535 * 16) blocks = 65535 * 16;
+  dim3 grid((unsigned)blocks), block(256);
+  if (delta_dtype == PYLON_F32)
+    hipLaunchKernelGGL(add_kernel<float>, grid, block, 0, stream, resid, (const float*)delta, (size_t)count);
+  else
+    hipLaunchKernelGGL(add_kernel<bf16_t>, grid, block, 0, stream, resid, (const bf16_t*)delta,
+                       (size_t)count);
+  PYLON_LAUNCHED("residual_add");
+}
+
+// ---- gated activation -----------------------------------------------------------------
+// out[t, i] = silu(gu[t, i]) * gu[t, inter + i]; silu(z) = z / (1 + exp(-z)).
+template <typename T>
+__global__ void silu_gate_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter, size_t total) {
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (; i < total; i += step) {
+    const size_t t = i / inter;
+    const size_t c = i - t * inter;
+    const float g = to_float(gu[t * 2 * inter + c]);
+    const float u = to_float(gu[t * 2 * inter + inter + c]);
+    const float s = g / (1.0f + expf(-g));
+    out[i] = from_float<T>(s * u);
+  }
+}
+
+extern "C" int pylon_silu_gate(void* out, const void* gate_up, int dtype, int tokens, int inter,
+                               hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(dtype), "silu_gate: unknown dtype");
+  PYLON_REQUIRE(tokens >= 0 && inter > 0, "silu_gate: bad sizes tokens=%d inter=%d", tokens, inter);
+  const size_t total = static_cast<size_t>(tokens) * inter;
+  if (total == 0) return 0;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65535u * 16u) blocks = 65535u * 16u;
+  dim3 grid((unsigned)blocks), block(256);
+  if (dtype == PYLON_F32)
+    hipLaunchKernelGGL(silu_gate_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)gate_up,
+                       inter, total);
+  else
+    hipLaunchKernelGGL(silu_gate_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out,
+                       (const bf16_t*)gate_up, inter, total);
+  PYLON_LAUNCHED("silu_gate");
+}

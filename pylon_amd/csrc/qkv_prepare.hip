@@ -1,0 +1,124 @@
+// What happens between the fused q/k/v projection and attention, in one pass over the
+// projection's output: per-head RMSNorm of q and k (optional), rotary position encoding
+// of q and k (optional), q written out head-major, k and v scattered into their cache
+// pages.  One wavefront handles one head of one token.  Norm, angles and rotation are
+// computed in float and rounded once on the store.
+#include "common.h"
+
+#define QKV_WAVES 4
+
+template <typename T>
+__global__ void qkv_prepare_kernel(T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                   const T* __restrict__ qkv, long long row_stride,
+                                   const float* __restrict__ q_weight, const float* __restrict__ k_weight,
+                                   float eps, const float* __restrict__ inv_freq, int rot_dim,
+                                   const int* __restrict__ positions, const int* __restrict__ slot_map,
+                                   long long items, int n_heads, int n_kv_heads, int head_dim,
+                                   int heads_per_token) {
+  extern __shared__ float lds[];
+  const int lane = threadIdx.x & (PYLON_WAVE - 1);
+  const int wave = threadIdx.x / PYLON_WAVE;
+  float* buf = lds + wave * head_dim;
+  const long long item = static_cast<long long>(blockIdx.x) * QKV_WAVES + wave;
+  const bool active = item < items;
+
+  int t = 0, s = 0;
+  const T* src = nullptr;
+  T* dst = nullptr;
+  const float* weight = nullptr;
+  bool rotate = false;
+  if (active) {
+    t = static_cast<int>(item / heads_per_token);
+    s = static_cast<int>(item - static_cast<long long>(t) * heads_per_token);
+    const T* row = qkv + static_cast<size_t>(t) * row_stride;
+    if (s < n_heads) {
+      src = row + static_cast<size_t>(s) * head_dim;
+      dst = q_out + (static_cast<size_t>(t) * n_heads + s) * head_dim;
+      weight = q_weight;
+      rotate = inv_freq != nullptr;
+    } else {
+      const int slot = slot_map[t];
+      const int j = (s - n_heads) % n_kv_heads;
+      const bool is_key = (s - n_heads) < n_kv_heads;
+      src = row + (static_cast<size_t>(n_heads) + (is_key ? 0 : n_kv_heads) + j) * head_dim;
+      if (slot >= 0) {
+        T* base = is_key ? k_cache : v_cache;
+        dst = base + (static_cast<size_t>(slot) * n_kv_heads + j) * head_dim;
+      }
+      weight = is_key ? k_weight : nullptr;
+      rotate = is_key && inv_freq != nullptr;
+    }
+  }
+
+  float ss = 0.f;
+  if (active) {
+    for (int i = lane; i < head_dim; i += PYLON_WAVE) {
+      const float v = to_float(src[i]);
+      buf[i] = v;
+      ss += v * v;
+    }
+  }
+  ss = wave_sum(ss);
+  __syncthreads();
+  if (active && weight != nullptr) {
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(head_dim) + eps);
+    for (int i = lane; i < head_dim; i += PYLON_WAVE) buf[i] = (buf[i] * inv) * weight[i];
+  }
+  __syncthreads();
+  if (active && rotate) {
+    const int half = rot_dim / 2;
+    const float pos = static_cast<float>(positions[t]);
+    for (int i = lane; i < half; i += PYLON_WAVE) {
+      const float angle = pos * inv_freq[i];
+      const float c = cosf(angle);
+      const float sn = sinf(angle);
+      const float a = buf[i];
+      const float b = buf[i + half];
+      buf[i] = a * c - b * sn;
+      buf[i + half] = b * c + a * sn;
+    }
+  }
+  __syncthreads();
+  if (active && dst != nullptr) {
+    for (int i = lane; i < head_dim; i += PYLON_WAVE) dst[i] = from_float<T>(buf[i]);
+  }
+}
+
+// qkv: [tokens, row_stride] with q heads first, then (if store_kv) k heads, then v heads.
+// q_out: [tokens, n_heads, head_dim]. k_cache/v_cache: [slots, n_kv_heads, head_dim] where a
+// slot is page*page_size + offset; slot_map[t] < 0 stores nothing for token t.
+extern "C" int pylon_qkv_prepare(void* q_out, void* k_cache, void* v_cache, const void* qkv, int dtype,
+                                 long long row_stride, const float* q_weight, const float* k_weight,
+                                 float eps, const float* inv_freq, int rot_dim, const int* positions,
+                                 const int* slot_map, int tokens, int n_heads, int n_kv_heads,
+                                 int head_dim, int store_kv, hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(dtype), "qkv_prepare: unknown dtype");
+  PYLON_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0, "qkv_prepare: bad head counts");
+  PYLON_REQUIRE(head_dim > 0 && head_dim <= 1024, "qkv_prepare: head_dim %d is outside 1..1024", head_dim);
+  const int heads_per_token = n_heads + (store_kv ? 2 * n_kv_heads : 0);
+  PYLON_REQUIRE(row_stride >= static_cast<long long>(heads_per_token) * head_dim,
+                "qkv_prepare: row stride %lld is shorter than %d heads of %d", row_stride,
+                heads_per_token, head_dim);
+  if (inv_freq != nullptr) {
+    PYLON_REQUIRE(rot_dim > 0 && rot_dim % 2 == 0 && rot_dim <= head_dim,
+                  "qkv_prepare: rotary dim %d must be even and at most head_dim %d", rot_dim, head_dim);
+    PYLON_REQUIRE(positions != nullptr, "qkv_prepare: rotary encoding needs positions");
+  }
+  if (store_kv) PYLON_REQUIRE(k_cache && v_cache && slot_map, "qkv_prepare: storing k/v needs the cache and a slot map");
+  if (tokens == 0) return 0;
+  const long long items = static_cast<long long>(tokens) * heads_per_token;
+  const long long blocks = (items + QKV_WAVES - 1) / QKV_WAVES;
+  PYLON_REQUIRE(blocks < (1ll << 31), "qkv_prepare: too many heads to process in one launch");
+  dim3 grid((unsigned)blocks), block(QKV_WAVES * PYLON_WAVE);
+  const size_t lds = sizeof(float) * QKV_WAVES * head_dim;
+  if (dtype == PYLON_F32)
+    hipLaunchKernelGGL(qkv_prepare_kernel<float>, grid, block, lds, stream, (float*)q_out, (float*)k_cache,
+                       (float*)v_cache, (const float*)qkv, row_stride, q_weight, k_weight, eps, inv_freq,
+                       rot_dim, positions, slot_map, items, n_heads, n_kv_heads, head_dim, heads_per_token);
+  else
+    hipLaunchKernelGGL(qkv_prepare_kernel<bf16_t>, grid, block, lds, stream, (bf16_t*)q_out,
+                       (bf16_t*)k_cache, (bf16_t*)v_cache, (const bf16_t*)qkv, row_stride, q_weight,
+                       k_weight, eps, inv_freq, rot_dim, positions, slot_map, items, n_heads, n_kv_heads,
+                       head_dim, heads_per_token);
+  PYLON_LAUNCHED("qkv_prepare");
+}

@@ -1,0 +1,211 @@
+"""One step's batch: which tokens of which requests run, and everything the kernels
+need to know about them, as one packed block of int32 that crosses to the device in a
+single copy.
+
+The vectors are the ones the reference builds in ``PackedBatchCache.prepare_packed``
+(/root/reference/src/pylon/kv/cache.py:409-450): token ids, positions, the prefix sums
+of the rows' token counts (its ``cu_seq_q``), the rows' lengths after the step (its
+``seqused_k``), the block table, the cache slot of every token (its ``write_slots``) and
+the indices whose logits are wanted (its ``last_indices``).  The reference fills them
+with Python loops over every token; here they are numpy gathers.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence as Seq, Tuple
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager, CacheView, Sequence
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step: its next tokens and which of them need logits."""
+
+    seq: Sequence
+    tokens: Seq[int]
+    want: Seq[int] = ()  # indices into `tokens`
+
+
+def _align4(n: int) -> int:
+    return (n + 3) & ~3
+
+
+class MetadataArena:
+    """Pinned host buffers (used in rotation) and one device buffer for step metadata."""
+
+    def __init__(self, device, capacity: int = 1 << 16, rotation: int = 4) -> None:
+        self.device = torch.device(device)
+        self.rotation = rotation
+        self._cursor = 0
+        self._capacity = 0
+        self._host: List[torch.Tensor] = []
+        self._events: List[Optional[torch.cuda.Event]] = []
+        self._device_buf: Optional[torch.Tensor] = None
+        self._grow(capacity)
+
+    def _grow(self, capacity: int) -> None:
+        pin = self.device.type == "cuda"
+        if pin:
+            torch.cuda.synchronize(self.device)
+        self._capacity = capacity
+        self._host = [torch.empty(capacity, dtype=torch.int32, pin_memory=pin) for _ in range(self.rotation)]
+        self._events = [None] * self.rotation
+        self._device_buf = torch.empty(capacity, dtype=torch.int32, device=self.device)
+
+    def acquire(self, size: int) -> Tuple[np.ndarray, int]:
+        """A host buffer of at least ``size`` ints that no pending copy still reads."""
+        if size > self._capacity:
+            self._grow(max(size, 2 * self._capacity))
+        index = self._cursor
+        self._cursor = (self._cursor + 1) % self.rotation
+        event = self._events[index]
+        if event is not None:
+            event.synchronize()
+        return self._host[index].numpy(), index
+
+    def upload(self, index: int, size: int, into: Optional[torch.Tensor] = None) -> torch.Tensor:
+        target = self._device_buf if into is None else into
+        target[:size].copy_(self._host[index][:size], non_blocking=True)
+        if self.device.type == "cuda":
+            event = torch.cuda.Event()
+            event.record()
+            self._events[index] = event
+        return target
+
+
+@dataclass
+class StepContext:
+    """What parts see of the running step."""
+
+    tokens: int
+    rows: int
+    token_ids: torch.Tensor  # int32 [tokens]
+    positions: torch.Tensor  # int32 [tokens]: index of each token in its request
+    tok_row: torch.Tensor  # int32 [tokens]: row (request of this step) of each token
+    row_start: torch.Tensor  # int32 [rows + 1]: prefix sums of the rows' token counts
+    seq_lens: torch.Tensor  # int32 [rows]: cached length of each row after this step
+    row_slots: torch.Tensor  # int32 [rows]: state slot of each row's request
+    row_first: torch.Tensor  # int32 [rows]: 1 where the row's tokens start its request
+    logit_idx: Optional[torch.Tensor]  # int32 [n]: token indices whose logits are wanted
+    n_logits: int
+    views: Dict[int, CacheView]
+    # host-side copies for parts that plan their launches on the host
+    counts: np.ndarray = field(default=None)
+    starts: np.ndarray = field(default=None)
+    max_count: int = 0
+    max_len: int = 0
+    decode_only: bool = False
+
+    def cache(self, cache_id: int) -> CacheView:
+        return self.views[cache_id]
+
+
+def plan_layout(tokens: int, rows: int, n_logits: int, n_groups: int, width: int) -> Tuple[Dict[str, Tuple[int, int]], int]:
+    """Offsets (in int32 units, each a multiple of 4) of every vector in the packed block."""
+    layout: Dict[str, Tuple[int, int]] = {}
+    cursor = 0
+
+    def put(name: str, size: int) -> None:
+        nonlocal cursor
+        layout[name] = (cursor, size)
+        cursor += _align4(max(size, 1))
+
+    put("token_ids", tokens)
+    put("positions", tokens)
+    put("tok_row", tokens)
+    put("row_start", rows + 1)
+    put("seq_lens", rows)
+    put("row_slots", rows)
+    put("row_first", rows)
+    put("logit_idx", n_logits)
+    for g in range(n_groups):
+        put(f"slot_map{g}", tokens)
+        put(f"block_table{g}", rows * width)
+    return layout, cursor
+
+
+def build_step(entries: Seq[StepEntry], manager: CacheManager, arena: MetadataArena, *,
+               vocab_size: int, width: Optional[int] = None,
+               device_block: Optional[torch.Tensor] = None) -> StepContext:
+    """Check the entries, take the pages they need, and put the step's metadata on the
+    device.  Raises before touching the cache if any entry is malformed; raises
+    :class:`~pylon_amd.cache.pages.OutOfPages` (cache untouched) if pages run short."""
+    if not entries:
+        raise ValueError("a step needs at least one entry")
+    rows = len(entries)
+    counts = np.fromiter((len(e.tokens) for e in entries), dtype=np.int64, count=rows)
+    if (counts < 1).any():
+        raise ValueError("Each packed sequence needs at least one query token.")
+    tokens = int(counts.sum())
+    flat = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+    if flat.size and (flat.min() < 0 or flat.max() >= vocab_size):
+        raise ValueError(f"Token IDs must be between 0 and {vocab_size - 1:,}.")
+    row_start = np.zeros(rows + 1, dtype=np.int64)
+    np.cumsum(counts, out=row_start[1:])
+    logit_list: List[int] = []
+    for r, e in enumerate(entries):
+        for w in e.want:
+            if not 0 <= w < counts[r]:
+                raise ValueError(f"wanted index {w} is outside the {counts[r]} tokens of its entry")
+            logit_list.append(int(row_start[r]) + int(w))
+    pairs = [(e.seq, int(c)) for e, c in zip(entries, counts)]
+    manager.reserve(pairs)  # all-or-nothing
+
+    starts = np.fromiter((e.seq.length for e in entries), dtype=np.int64, count=rows)
+    slots = np.fromiter((e.seq.slot for e in entries), dtype=np.int64, count=rows)
+    tok_row = np.repeat(np.arange(rows, dtype=np.int64), counts)
+    positions = starts[tok_row] + (np.arange(tokens, dtype=np.int64) - row_start[tok_row])
+    seq_lens = starts + counts
+    need_width = int(-(-seq_lens.max() // manager.page_size))
+    if width is None:
+        width = need_width
+    elif need_width > width:
+        manager.cancel(pairs)
+        raise ValueError(f"a request needs {need_width} pages but the block table holds {width}")
+
+    n_groups = len(manager.groups)
+    layout, size = plan_layout(tokens, rows, len(logit_list), n_groups, width)
+    host, index = arena.acquire(size)
+
+    def seg(name: str) -> np.ndarray:
+        off, n = layout[name]
+        return host[off: off + n]
+
+    seg("token_ids")[:] = flat
+    seg("positions")[:] = positions
+    seg("tok_row")[:] = tok_row
+    seg("row_start")[:] = row_start
+    seg("seq_lens")[:] = seq_lens
+    seg("row_slots")[:] = slots
+    seg("row_first")[:] = starts == 0
+    if logit_list:
+        seg("logit_idx")[:] = logit_list
+    token_slots = slots[tok_row]
+    for g in range(n_groups):
+        manager.slot_map(g, token_slots, positions, seg(f"slot_map{g}"))
+        manager.block_table(g, slots, width, seg(f"block_table{g}").reshape(rows, width))
+    block = arena.upload(index, size, into=device_block)
+
+    def dev(name: str) -> torch.Tensor:
+        off, n = layout[name]
+        return block[off: off + n]
+
+    views: Dict[int, CacheView] = {}
+    for cache_id in range(manager.n_caches):
+        view = manager.view(cache_id)
+        if view.group >= 0:
+            view.slot_map = dev(f"slot_map{view.group}")
+            view.block_table = dev(f"block_table{view.group}").view(rows, width)
+        views[cache_id] = view
+    return StepContext(
+        tokens=tokens, rows=rows,
+        token_ids=dev("token_ids"), positions=dev("positions"), tok_row=dev("tok_row"),
+        row_start=dev("row_start"), seq_lens=dev("seq_lens"), row_slots=dev("row_slots"),
+        row_first=dev("row_first"),
+        logit_idx=dev("logit_idx") if logit_list else None, n_logits=len(logit_list),
+        views=views, counts=counts, starts=starts, max_count=int(counts.max()),
+        max_len=int(seq_lens.max()), decode_only=bool((counts == 1).all()),
+    )

@@ -1,0 +1,89 @@
+"""A decoder assembled from parts, and its one forward pass: the step.
+
+The model is architecture-blind: it builds one block per :class:`LayerSpec`, runs the
+blocks in the order the schedule lists them, and applies the final norm and the
+vocabulary head only at the tokens whose logits are wanted
+(/root/reference/src/pylon/model/model.py:124-144).
+"""
+from __future__ import annotations
+
+from typing import Dict, Iterator, List, Optional, Tuple
+
+import torch
+
+from ..config.specs import ModelSpec
+from ..kernels import ops
+from ..parts import build_part
+from ..parts.base import Part
+from .batch import StepContext
+
+
+class Model(Part):
+    def __init__(self, spec: ModelSpec, *, dtype: torch.dtype, device) -> None:
+        super().__init__()
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError("the model runs in float32 or bfloat16")
+        self.spec = spec
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.schedule = spec.resolved_schedule()
+        self.add_param("embed", (spec.vocab_size, spec.hidden_size), dtype, device)
+        if not spec.tie_word_embeddings:
+            self.add_param("lm_head", (spec.vocab_size, spec.hidden_size), dtype, device)
+        self.blocks: List[Part] = []
+        for index, layer in enumerate(spec.layers):
+            block = build_part("block", layer, dtype=dtype, device=device)
+            self.blocks.append(block)
+            self.add_child(f"layers.{index}", block)
+        self.final_norm = self.add_child(
+            "final_norm", build_part("norm", spec.final_norm, dtype=dtype, device=device)
+        )
+
+    # ---- what the cache manager has to provide ------------------------------------------
+    def cache_requirements(self) -> List[object]:
+        """Per run of the schedule: what its mixer keeps (None for a run that borrows)."""
+        needs: List[object] = []
+        for layer, cache_id, stores in self.schedule:
+            needs.append(self.blocks[layer].cache_requirement() if stores else None)
+        for index, (layer, cache_id, stores) in enumerate(self.schedule):
+            if not stores:
+                own = self.blocks[layer].cache_requirement()
+                if own != needs[cache_id]:
+                    raise ValueError(
+                        f"run {index} borrows the cache of run {cache_id}, which has another geometry"
+                    )
+        return needs
+
+    @property
+    def head_weight(self) -> torch.Tensor:
+        return self.params["embed"] if self.spec.tie_word_embeddings else self.params["lm_head"]
+
+    # ---- the step --------------------------------------------------------------------------
+    def step(self, ctx: StepContext) -> Optional[torch.Tensor]:
+        """Run the step's tokens through every scheduled layer, from and into the cache.
+        Returns float32 logits ``[n_logits, vocab]`` (None when no logits are wanted)."""
+        resid = ops.embed(ctx.token_ids, self.params["embed"], scale=self.spec.embedding_scale)
+        delta = None
+        for layer, cache_id, stores in self.schedule:
+            resid, delta = self.blocks[layer].forward(resid, delta, ctx, ctx.cache(cache_id), stores)
+        if ctx.n_logits == 0:
+            return None
+        h = self.final_norm.add_forward(resid, delta, row_idx=ctx.logit_idx)
+        return ops.linear(h, self.head_weight, out_dtype=torch.float32)
+
+    # ---- random weights in place (for measurements at sizes not worth writing to disk) ----
+    def init_random(self, seed: int, std: float = 0.02) -> None:
+        gen = torch.Generator(device=self.device)
+        gen.manual_seed(seed)
+        for path, owner, name in self.named_params():
+            tensor = owner.params[name]
+            if owner.param_roles[name] == "vector":
+                tensor.fill_(1.0)
+            else:
+                # Drawn in slabs so that no float32 copy of a large matrix is needed.
+                flat = tensor.view(-1)
+                step = 1 << 26
+                for start in range(0, flat.numel(), step):
+                    part = flat[start: start + step]
+                    part.copy_(torch.randn(part.numel(), generator=gen, device=self.device,
+                                           dtype=torch.float32) * std)

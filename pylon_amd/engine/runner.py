@@ -1,0 +1,93 @@
+"""The step executor: a model, its cache manager, and the one step function.
+
+It plays the part of the reference's ``Decoder``
+(/root/reference/src/pylon/decode/runner.py:58-302): it owns the page pool, opens and
+releases request caches, and runs packed batches.  Unlike the reference there is one
+step function for every kind of batch; a decode-only step differs only in that it may
+be replayed from a HIP graph.
+"""
+from __future__ import annotations
+
+from pathlib import Path
+from typing import Hashable, List, Optional, Sequence as Seq
+
+import torch
+
+from ..cache.manager import CacheManager, Sequence
+from ..config.registry import load_model_config
+from ..kernels import check_device
+from ..weights.loader import load_weights
+from .batch import MetadataArena, StepEntry, build_step
+from .model import Model
+
+_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32,
+           torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+def resolve_dtype(dtype) -> torch.dtype:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise ValueError("dtype must be bfloat16 or float32") from None
+
+
+class Runner:
+    def __init__(self, model: Model, *, page_size: int, num_pages: int, max_requests: int) -> None:
+        if model.device.type != "cuda":
+            raise RuntimeError("A GPU is required: the step function has no CPU path.")
+        check_device()
+        self.model = model
+        self.manager = CacheManager(
+            model.cache_requirements(), page_size=page_size, num_pages=num_pages,
+            max_requests=max_requests, dtype=model.dtype, device=model.device,
+        )
+        self.arena = MetadataArena(model.device)
+        self.graphs = None
+
+    # ---- construction ------------------------------------------------------------------
+    @classmethod
+    def from_folder(cls, folder, *, dtype="bfloat16", device="cuda:0", page_size: int = 256,
+                    num_pages: int, max_requests: int = 32) -> "Runner":
+        """Load the model folder ``folder`` (config.json decides the model class)."""
+        if not torch.cuda.is_available():
+            raise RuntimeError("A GPU is required: the step function has no CPU path.")
+        arch, config = load_model_config(folder)
+        model = Model(arch.model_spec(config), dtype=resolve_dtype(dtype), device=device)
+        load_weights(model, arch, config, Path(folder))
+        runner = cls(model, page_size=page_size, num_pages=num_pages, max_requests=max_requests)
+        runner.config = config
+        return runner
+
+    # ---- requests -------------------------------------------------------------------------
+    def open(self, request_id: Hashable, capacity: Optional[int] = None) -> Sequence:
+        max_positions = self.model.spec.max_positions
+        if capacity is not None and max_positions and capacity > max_positions:
+            raise ValueError(
+                f"KV-cache capacity must be between 1 and {max_positions:,} tokens."
+            )
+        return self.manager.open(request_id, capacity)
+
+    def close(self, seq: Sequence) -> None:
+        self.manager.close(seq)
+
+    # ---- the step ---------------------------------------------------------------------------
+    def step(self, entries: Seq[StepEntry]) -> Optional[torch.Tensor]:
+        """Run the given tokens of the given requests as one batch, from the cache that
+        earlier steps left, and return float32 logits at the wanted places (in the order
+        of the entries and of their ``want``), or None if nothing is wanted."""
+        max_positions = self.model.spec.max_positions
+        if max_positions:
+            for e in entries:
+                if e.seq.length + len(e.tokens) > max_positions:
+                    raise ValueError(
+                        f"The model supports at most {max_positions:,} tokens per request."
+                    )
+        ctx = build_step(entries, self.manager, self.arena, vocab_size=self.model.spec.vocab_size)
+        pairs = [(e.seq, len(e.tokens)) for e in entries]
+        try:
+            logits = self.model.step(ctx)
+        except Exception:
+            self.manager.cancel(pairs)
+            raise
+        self.manager.commit(pairs)
+        return logits

@@ -1,0 +1,264 @@
+"""Tensor-level wrappers of the HIP entry points.
+
+Every wrapper checks device, element type, contiguity and shapes on the host before
+it launches, and launches on torch's current stream.  None has a CPU path.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import library as _lib
+from .library import KernelError
+
+F32 = 0
+BF16 = 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise KernelError(f"the kernels take float32 and bfloat16, not {dtype}") from None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: Optional[torch.Tensor], name: str, dtype=None) -> int:
+    """Device pointer of a checked tensor (0 for None)."""
+    if t is None:
+        return 0
+    if not t.is_cuda:
+        raise KernelError(f"{name} must live on the GPU; there is no CPU path")
+    if not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, got {t.dtype}")
+    return t.data_ptr()
+
+
+def embed(ids: torch.Tensor, table: torch.Tensor, *, scale: float = 1.0,
+          out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 ``out[t] = table[ids[t]] * scale``."""
+    tokens = ids.numel()
+    vocab, hidden = table.shape
+    if out is None:
+        out = torch.empty((tokens, hidden), dtype=torch.float32, device=table.device)
+    elif out.shape != (tokens, hidden):
+        raise KernelError(f"embed: out has shape {tuple(out.shape)}, expected {(tokens, hidden)}")
+    _lib.call("pylon_embed", _dev(out, "out", torch.float32), _dev(table, "table"),
+              dtype_code(table.dtype), _dev(ids, "ids", torch.int32), tokens, hidden, vocab,
+              float(scale), _stream())
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, *, out_dtype=None,
+            row_idx: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``(x / sqrt(mean(x^2) + eps)) * weight`` over the last axis of a 2-D tensor."""
+    if x.dim() != 2:
+        raise KernelError("rmsnorm takes a 2-D input")
+    dim = x.shape[1]
+    if weight.shape != (dim,):
+        raise KernelError(f"rmsnorm: weight has shape {tuple(weight.shape)}, expected ({dim},)")
+    rows = x.shape[0] if row_idx is None else row_idx.numel()
+    out_dtype = out_dtype or x.dtype
+    if out is None:
+        out = torch.empty((rows, dim), dtype=out_dtype, device=x.device)
+    elif out.shape != (rows, dim):
+        raise KernelError("rmsnorm: out has the wrong shape")
+    _lib.call("pylon_rmsnorm", _dev(out, "out"), dtype_code(out.dtype), _dev(x, "x"),
+              dtype_code(x.dtype), _dev(weight, "weight", torch.float32),
+              _dev(row_idx, "row_idx", torch.int32), rows, dim, float(eps), _stream())
+    return out
+
+
+def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, *, row_idx: Optional[torch.Tensor] = None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``resid += delta`` (float32, in place) and the RMSNorm of the sum.
+
+    With ``row_idx`` only those rows are normed and ``resid`` is left as it is.
+    """
+    if resid.dim() != 2:
+        raise KernelError("add_rmsnorm takes a 2-D residual")
+    dim = resid.shape[1]
+    if delta is not None and delta.shape != resid.shape:
+        raise KernelError("add_rmsnorm: delta and resid differ in shape")
+    if weight.shape != (dim,):
+        raise KernelError(f"add_rmsnorm: weight has shape {tuple(weight.shape)}, expected ({dim},)")
+    rows = resid.shape[0] if row_idx is None else row_idx.numel()
+    if out is None:
+        out = torch.empty((rows, dim), dtype=out_dtype, device=resid.device)
+    elif out.shape != (rows, dim) or out.dtype != out_dtype:
+        raise KernelError("add_rmsnorm: out has the wrong shape or dtype")
+    _lib.call("pylon_add_rmsnorm", _dev(out, "out"), dtype_code(out.dtype),
+              _dev(resid, "resid", torch.float32), _dev(delta, "delta"),
+              dtype_code(delta.dtype) if delta is not None else F32,
+              _dev(weight, "weight", torch.float32), _dev(row_idx, "row_idx", torch.int32),
+              rows, dim, float(eps), _stream())
+    return out
+
+
+def residual_add(resid: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    if delta.shape != resid.shape:
+        raise KernelError("residual_add: shapes differ")
+    _lib.call("pylon_residual_add", _dev(resid, "resid", torch.float32), _dev(delta, "delta"),
+              dtype_code(delta.dtype), resid.numel(), _stream())
+    return resid
+
+
+def silu_gate(gate_up: torch.Tensor, *, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``silu(gate_up[:, :I]) * gate_up[:, I:]`` for a ``[tokens, 2I]`` input."""
+    if gate_up.dim() != 2 or gate_up.shape[1] % 2:
+        raise KernelError("silu_gate takes a [tokens, 2*I] input")
+    tokens, two_i = gate_up.shape
+    inter = two_i // 2
+    if out is None:
+        out = torch.empty((tokens, inter), dtype=gate_up.dtype, device=gate_up.device)
+    elif out.shape != (tokens, inter) or out.dtype != gate_up.dtype:
+        raise KernelError("silu_gate: out has the wrong shape or dtype")
+    _lib.call("pylon_silu_gate", _dev(out, "out"), _dev(gate_up, "gate_up"),
+              dtype_code(gate_up.dtype), tokens, inter, _stream())
+    return out
+
+
+def qkv_prepare(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: Optional[torch.Tensor],
+                v_cache: Optional[torch.Tensor], *, n_heads: int, n_kv_heads: int, head_dim: int,
+                q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                inv_freq: Optional[torch.Tensor], rot_dim: int, positions: Optional[torch.Tensor],
+                slot_map: Optional[torch.Tensor], store_kv: bool) -> None:
+    """Per-head norm and rotation of q and k; q to ``q_out``; k and v into cache slots."""
+    if qkv.dim() != 2:
+        raise KernelError("qkv_prepare takes a 2-D projection output")
+    tokens, width = qkv.shape
+    heads = n_heads + (2 * n_kv_heads if store_kv else 0)
+    if width != heads * head_dim:
+        raise KernelError(f"qkv_prepare: projection width {width} is not {heads} heads of {head_dim}")
+    if q_out.shape != (tokens, n_heads, head_dim) or q_out.dtype != qkv.dtype:
+        raise KernelError("qkv_prepare: q_out has the wrong shape or dtype")
+    for name, wt in (("q_weight", q_weight), ("k_weight", k_weight)):
+        if wt is not None and wt.shape != (head_dim,):
+            raise KernelError(f"qkv_prepare: {name} must have shape ({head_dim},)")
+    if inv_freq is not None and inv_freq.numel() != rot_dim // 2:
+        raise KernelError("qkv_prepare: inv_freq must hold rot_dim/2 frequencies")
+    if positions is not None and positions.numel() != tokens:
+        raise KernelError("qkv_prepare: one position per token is required")
+    if store_kv:
+        if k_cache is None or v_cache is None or slot_map is None:
+            raise KernelError("qkv_prepare: storing needs k_cache, v_cache and slot_map")
+        if slot_map.numel() != tokens:
+            raise KernelError("qkv_prepare: one cache slot per token is required")
+        for name, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+            if c.dtype != qkv.dtype or c.shape[-2:] != (n_kv_heads, head_dim):
+                raise KernelError(f"qkv_prepare: {name} must be [..., {n_kv_heads}, {head_dim}] of {qkv.dtype}")
+    _lib.call("pylon_qkv_prepare", _dev(q_out, "q_out"), _dev(k_cache if store_kv else None, "k_cache"),
+              _dev(v_cache if store_kv else None, "v_cache"), _dev(qkv, "qkv"), dtype_code(qkv.dtype),
+              width, _dev(q_weight, "q_weight", torch.float32), _dev(k_weight, "k_weight", torch.float32),
+              float(eps), _dev(inv_freq, "inv_freq", torch.float32), int(rot_dim),
+              _dev(positions, "positions", torch.int32), _dev(slot_map if store_kv else None, "slot_map", torch.int32),
+              tokens, n_heads, n_kv_heads, head_dim, 1 if store_kv else 0, _stream())
+
+
+def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                    block_table: torch.Tensor, tok_row: torch.Tensor, positions: torch.Tensor, *,
+                    page_size: int, window: Optional[int], scale: float,
+                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal attention of each token over its request's cached keys ``<=`` its position."""
+    if q.dim() != 3:
+        raise KernelError("paged_attention takes q as [tokens, heads, head_dim]")
+    tokens, n_heads, head_dim = q.shape
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape:
+        raise KernelError("paged_attention: caches must be [pages, page_size, kv_heads, head_dim]")
+    pages, psize, n_kv_heads, hd = k_cache.shape
+    if psize != page_size or hd != head_dim:
+        raise KernelError("paged_attention: cache geometry does not match page_size/head_dim")
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        raise KernelError("paged_attention: q and the caches differ in dtype")
+    if pages * page_size >= 2 ** 31:
+        raise KernelError("paged_attention: the cache holds more slots than an int32 can index")
+    if block_table.dim() != 2:
+        raise KernelError("paged_attention: block_table must be [rows, width]")
+    if tok_row.numel() != tokens or positions.numel() != tokens:
+        raise KernelError("paged_attention: one row id and one position per token are required")
+    if out is None:
+        out = torch.empty_like(q)
+    elif out.shape != q.shape or out.dtype != q.dtype:
+        raise KernelError("paged_attention: out has the wrong shape or dtype")
+    _lib.call("pylon_paged_attention", _dev(out, "out"), _dev(q, "q"), _dev(k_cache, "k_cache"),
+              _dev(v_cache, "v_cache"), dtype_code(q.dtype), _dev(block_table, "block_table", torch.int32),
+              block_table.shape[1], _dev(tok_row, "tok_row", torch.int32),
+              _dev(positions, "positions", torch.int32), tokens, n_heads, n_kv_heads, head_dim,
+              page_size, int(window or 0), float(scale), _stream())
+    return out
+
+
+def gemm_tiled(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.dtype] = None,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x @ weight.T`` with float accumulation on the vector units (no matrix cores)."""
+    if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
+        raise KernelError(f"gemm: cannot multiply {tuple(x.shape)} by the transpose of {tuple(weight.shape)}")
+    m, k = x.shape
+    n = weight.shape[0]
+    out_dtype = out_dtype or x.dtype
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    elif out.shape != (m, n):
+        raise KernelError("gemm: out has the wrong shape")
+    if x.stride(1) != 1 or weight.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("gemm: rows must be contiguous")
+    for name, t in (("x", x), ("weight", weight), ("out", out)):
+        if not t.is_cuda:
+            raise KernelError(f"gemm: {name} must live on the GPU; there is no CPU path")
+    _lib.call("pylon_gemm_tiled", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), dtype_code(x.dtype),
+              weight.data_ptr(), dtype_code(weight.dtype), m, n, k, x.stride(0), weight.stride(0),
+              out.stride(0), _stream())
+    return out
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``x @ weight.T``.
+
+    bfloat16 by bfloat16 goes to the library matrix product (as the reference's
+    ``nn.Linear`` does); every pairing that involves float32 operands runs on the
+    exact tiled kernel, which never uses a reduced-precision matrix mode.
+    """
+    out_dtype = out_dtype or x.dtype
+    if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
+        if not x.is_cuda:
+            raise KernelError("linear: operands must live on the GPU; there is no CPU path")
+        y = torch.nn.functional.linear(x, weight)
+        return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
+    return gemm_tiled(x, weight, out_dtype=out_dtype)
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    if logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("argmax takes [rows, vocab] logits with contiguous rows")
+    rows, vocab = logits.shape
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    if not logits.is_cuda or logits.dtype != torch.float32:
+        raise KernelError("argmax takes float32 logits on the GPU")
+    _lib.call("pylon_argmax", out.data_ptr(), logits.data_ptr(), rows, vocab, logits.stride(0), _stream())
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
+           uniform: torch.Tensor) -> torch.Tensor:
+    """One token per row; rows with temperature 0 take the argmax."""
+    if logits.dim() != 2 or logits.stride(1) != 1:
+        raise KernelError("sample takes [rows, vocab] logits with contiguous rows")
+    rows, vocab = logits.shape
+    if not logits.is_cuda or logits.dtype != torch.float32:
+        raise KernelError("sample takes float32 logits on the GPU")
+    for name, t in (("temperature", temperature), ("top_p", top_p), ("uniform", uniform)):
+        if t.numel() != rows:
+            raise KernelError(f"sample: {name} must have one value per row")
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    _lib.call("pylon_sample", out.data_ptr(), logits.data_ptr(), rows, vocab, logits.stride(0),
+              _dev(temperature, "temperature", torch.float32), _dev(top_p, "top_p", torch.float32),
+              _dev(uniform, "uniform", torch.float32), _stream())
+    return out

@@ -1,0 +1,72 @@
+"""What every part of a layer looks like to the model that assembles it.
+
+A part owns named parameters (device tensors the weight loader fills by path) and a
+``forward``.  It gets its sizes and constants from its spec and the batch from the
+step context; it does not know which model, or which layer of it, it sits in.
+
+Interfaces
+----------
+norm          ``forward(x) -> y`` and ``add_forward(resid, delta, row_idx=None) -> y``:
+              ``resid`` is the float32 residual stream, ``delta`` the previous part's
+              output (or None); the sum is formed in float32, stored back into
+              ``resid`` (unless ``row_idx`` picks rows), and its norm is returned in
+              the activation dtype.
+position      ``rotary() -> (inv_freq, rotary_dim) | None`` for encodings applied by
+              rotating q and k, and ``check(max_position)``.
+mixer         ``cache_requirement() -> KVRequirement | StateRequirement | None`` and
+              ``forward(h, ctx, cache, stores) -> [tokens, hidden]``: ``cache`` is the
+              view of the run's cache (its own, or the one it borrows); ``stores``
+              says whether this run writes it.
+feed_forward  ``forward(h, ctx) -> [tokens, hidden]``.
+block         ``forward(resid, delta, ctx, cache, stores) -> (resid, delta)``: takes and
+              returns the residual stream and the not-yet-added output of the last part.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Iterator, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class KVRequirement:
+    """A growing cache of keys and values: one entry per token, in pages.
+
+    Runs whose requirements are equal share a group of pages (one block table)."""
+
+    n_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None  # keep only the last `window` tokens' entries
+
+
+@dataclass(frozen=True)
+class StateRequirement:
+    """Per-request state of fixed size, overwritten in place by every step."""
+
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    """Base of all parts: a bag of named parameters and named sub-parts."""
+
+    def __init__(self) -> None:
+        self.params: Dict[str, torch.Tensor] = {}
+        self.param_roles: Dict[str, str] = {}
+        self.children: Dict[str, "Part"] = {}
+
+    def add_param(self, name: str, shape, dtype: torch.dtype, device, role: str = "matrix") -> None:
+        self.params[name] = torch.empty(tuple(shape), dtype=dtype, device=device)
+        self.param_roles[name] = role
+
+    def add_child(self, name: str, part: "Part") -> "Part":
+        self.children[name] = part
+        return part
+
+    def named_params(self, prefix: str = "") -> Iterator[Tuple[str, "Part", str]]:
+        """``(path, owner, name)`` of every parameter below this part."""
+        for name in self.params:
+            yield prefix + name, self, name
+        for child_name, child in self.children.items():
+            yield from child.named_params(prefix + child_name + ".")
