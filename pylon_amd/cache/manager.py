@@ -33,6 +33,12 @@ def pages_for(tokens: int, page_size: int) -> int:
     return (tokens + page_size - 1) // page_size
 
 
+def bytes_per_token(requirements: Seq[object], dtype: torch.dtype) -> int:
+    """Cache bytes one token takes over all runs that keep keys and values."""
+    elem = torch.empty((), dtype=dtype).element_size()
+    return sum(2 * r.n_kv_heads * r.head_dim * elem for r in requirements if isinstance(r, KVRequirement))
+
+
 class KVGroup:
     """Runs with one key/value geometry: a pool of page ids and one K and V tensor per run."""
 

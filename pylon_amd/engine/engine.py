@@ -1,0 +1,451 @@
+"""The engine: the programming entry point on token ids.
+
+``Engine.enqueue(input_ids, eos_token_id, sampling, request_id) -> Future[GenerationResult]``
+has the reference's signature and meaning (/root/reference/src/pylon/engine.py:241-253);
+``generate`` is the same for a list of prompts, run to completion in the calling thread.
+A tick is the reference's (/root/reference/src/pylon/engine.py:255-300): drop cancelled
+requests, admit, run one step that carries every decoding request's pending token beside
+the prompt portions the token budget allows, sample where a row is ready, finish or
+continue each request, admit again into what was freed.
+"""
+from __future__ import annotations
+
+import logging
+import threading
+import time
+from collections import deque
+from concurrent.futures import Future
+from dataclasses import dataclass, field
+from typing import Callable, Deque, Iterable, List, Optional, Sequence, Tuple
+
+from ..cache.pages import OutOfPages
+from ..config.engine_config import PylonConfig
+from ..sampling.params import Sampling
+from .batch import StepEntry
+from .scheduler import AdmissionPolicy, PromptWork, Waiter, cut_prompts, hold_prompts
+
+logger = logging.getLogger("pylon")
+
+
+class QueueFullError(RuntimeError):
+    pass
+
+
+class EngineClosedError(RuntimeError):
+    pass
+
+
+@dataclass(frozen=True)
+class GenerationResult:
+    """/root/reference/src/pylon/engine.py:59-74, without the prefix-cache and
+    speculation fields."""
+
+    output_ids: List[int]
+    finish_reason: str  # "eos" or "length"
+    prefill_seconds: float
+    inter_token_seconds: List[float]
+    queue_seconds: float
+    first_token_seconds: Optional[float] = None
+    elapsed_seconds: Optional[float] = None
+
+
+@dataclass(frozen=True)
+class Request:
+    input_ids: List[int]
+    stop_ids: frozenset
+    sampling: Sampling
+    request_id: str
+
+
+@dataclass
+class Ticket:
+    """A request waiting for admission."""
+
+    request: Request
+    future: Future
+    arrived: float
+
+
+@dataclass
+class Active:
+    """A request that holds a cache: prefilling (no pending token) or decoding."""
+
+    ticket: Ticket
+    seq: object
+    reserved_pages: int
+    output_ids: List[int] = field(default_factory=list)
+    prompt_offset: int = 0
+    pending_token_id: Optional[int] = None
+    queue_seconds: float = 0.0
+    prefill_seconds: float = 0.0
+    inter_token_seconds: List[float] = field(default_factory=list)
+    prompt_wait_started: float = 0.0
+    first_token_at: Optional[float] = None
+
+    @property
+    def request(self) -> Request:
+        return self.ticket.request
+
+    @property
+    def remaining_prompt(self) -> int:
+        return len(self.request.input_ids) - self.prompt_offset
+
+
+def _stop_ids(eos_token_id) -> frozenset:
+    if eos_token_id is None:
+        return frozenset()
+    if isinstance(eos_token_id, int):
+        return frozenset((eos_token_id,))
+    return frozenset(eos_token_id)
+
+
+class Engine:
+    def __init__(self, config: PylonConfig, *, runner=None, sampler=None,
+                 clock: Callable[[], float] = time.perf_counter, threaded: bool = False) -> None:
+        """``runner`` executes steps (a :class:`~pylon_amd.engine.runner.Runner`; built from
+        ``config.model_path`` when not given).  ``threaded`` starts the background thread
+        that ticks on its own, as the reference's scheduler thread does; without it the
+        caller drives the engine with :meth:`tick`, :meth:`run_until_idle` or
+        :meth:`generate`."""
+        self._config = config
+        self._clock = clock
+        if runner is None:
+            runner = _load_runner(config)
+        self.runner = runner
+        if sampler is None:
+            from ..sampling.sampler import Sampler
+
+            sampler = Sampler(runner.model.device)
+        self.sampler = sampler
+        manager = runner.manager
+        self.page_size = manager.page_size
+        self.kv_budget_pages = manager.num_pages
+        self._policy = AdmissionPolicy(page_budget=manager.num_pages, page_size=manager.page_size,
+                                       admit_skip=config.admit_skip)
+        self._max_batch_size = config.max_batch_size
+        self._prefill_chunk_size = config.prefill_chunk_size
+        self._waiting: Deque[Ticket] = deque()
+        self._active: List[Active] = []
+        self._lock = threading.RLock()
+        self._wake = threading.Condition(self._lock)
+        self._closed = False
+        self.head_skips = 0
+        self._serial = 0
+        self.steps_run = 0
+        self.last_step = None  # (decode rows, prompt portions) of the most recent step
+        self._thread: Optional[threading.Thread] = None
+        if threaded:
+            self._thread = threading.Thread(target=self._drive, name="pylon-scheduler", daemon=True)
+            self._thread.start()
+
+    # ---- construction helpers ----------------------------------------------------------
+    @classmethod
+    def from_folder(cls, folder, **options) -> "Engine":
+        threaded = options.pop("threaded", False)
+        return cls(PylonConfig(model_path=str(folder), **options), threaded=threaded)
+
+    # ---- the public surface -------------------------------------------------------------
+    def enqueue(self, input_ids: Sequence[int], eos_token_id=None, sampling: Optional[Sampling] = None,
+                request_id: Optional[str] = None) -> Future:
+        sampling = sampling or Sampling()
+        request_id = request_id or "internal"
+        stop_ids = _stop_ids(eos_token_id)
+        input_ids = list(input_ids)
+        self._validate_request(input_ids, stop_ids, sampling)
+        ticket = Ticket(Request(input_ids, stop_ids, sampling, request_id), Future(), self._clock())
+        with self._wake:
+            if self._closed:
+                raise EngineClosedError("The generation scheduler is closed.")
+            self._sweep_cancelled_waiting()
+            if len(self._waiting) >= self._config.max_queue_size:
+                raise QueueFullError("The generation waiting queue is full.")
+            self._waiting.append(ticket)
+            self._wake.notify_all()
+        logger.info("request_waiting request_id=%s", request_id)
+        return ticket.future
+
+    def generate(self, prompts: Iterable[Sequence[int]], sampling: Optional[Sampling] = None,
+                 eos_token_id=None) -> List[GenerationResult]:
+        """Run the prompts to completion and return their results in order.  More prompts
+        than the queue holds are fed in as earlier ones finish."""
+        prompts = [list(p) for p in prompts]
+        futures: List[Optional[Future]] = [None] * len(prompts)
+        nxt = 0
+        while True:
+            while nxt < len(prompts) and len(self._waiting) < self._config.max_queue_size:
+                futures[nxt] = self.enqueue(prompts[nxt], eos_token_id, sampling, f"generate-{nxt}")
+                nxt += 1
+            if self._thread is not None:
+                break
+            busy = self.tick()
+            if not busy and nxt >= len(prompts):
+                break
+        if self._thread is not None:
+            for i in range(nxt, len(prompts)):
+                while len(self._waiting) >= self._config.max_queue_size:
+                    time.sleep(0.001)
+                futures[i] = self.enqueue(prompts[i], eos_token_id, sampling, f"generate-{i}")
+        return [f.result() for f in futures]
+
+    def run_until_idle(self) -> None:
+        while self.tick():
+            pass
+
+    def close(self) -> None:
+        with self._wake:
+            if self._closed:
+                return
+            self._closed = True
+            waiting, self._waiting = list(self._waiting), deque()
+            active, self._active = self._active, []
+            self._wake.notify_all()
+        error = EngineClosedError("The generation scheduler is closed.")
+        for item in active:
+            self.runner.close(item.seq)
+            if not item.ticket.future.done():
+                item.ticket.future.set_exception(error)
+        for ticket in waiting:
+            if not ticket.future.done():
+                ticket.future.set_exception(error)
+        if self._thread is not None and self._thread is not threading.current_thread():
+            self._thread.join()
+
+    def snapshot(self) -> dict:
+        with self._lock:
+            return {
+                "waiting": [t.request.request_id for t in self._waiting],
+                "active": [a.request.request_id for a in self._active],
+                "max_batch_size": self._max_batch_size,
+                "max_queue_size": self._config.max_queue_size,
+                "batch_wait_ms": self._config.batch_wait_ms,
+            }
+
+    # ---- page accounting ----------------------------------------------------------------
+    def request_cache_pages(self, token_count: int) -> int:
+        return self._policy.pages(token_count)
+
+    def reserved_pages(self) -> int:
+        return sum(item.reserved_pages for item in self._active)
+
+    # ---- one tick ---------------------------------------------------------------------------
+    def tick(self) -> bool:
+        """One round of admit, step, sample, finish.  True while work remains."""
+        with self._lock:
+            if self._closed:
+                return False
+            self._drop_cancelled_active()
+            self._admit()
+            if self._active:
+                try:
+                    self._run_step()
+                except Exception as error:
+                    logger.exception("model_batch_failed")
+                    self._fail_active(error)
+            self._admit()
+            return bool(self._active or self._waiting)
+
+    # ---- admission ----------------------------------------------------------------------------
+    def _sweep_cancelled_waiting(self) -> None:
+        if any(t.future.cancelled() for t in self._waiting):
+            self._waiting = deque(t for t in self._waiting if not t.future.cancelled())
+
+    def _admit(self) -> None:
+        while len(self._active) < self._max_batch_size:
+            self._sweep_cancelled_waiting()
+            if not self._waiting:
+                return
+            waiters = [
+                Waiter(t, len(t.request.input_ids) + t.request.sampling.max_new_tokens, t.arrived)
+                for t in self._waiting
+            ]
+            decoding = sum(1 for a in self._active if a.pending_token_id is not None)
+            verdict = self._policy.next(waiters, reserved_pages=self.reserved_pages(),
+                                        decoding=decoding, now=self._clock())
+            if verdict is None:
+                logger.info("continuous_admission_blocked request_id=%s reason=memory",
+                            self._waiting[0].request.request_id)
+                return
+            ticket: Ticket = verdict.key
+            self._waiting.remove(ticket)
+            if not ticket.future.set_running_or_notify_cancel():
+                continue
+            if not verdict.admit:
+                ticket.future.set_exception(RuntimeError(verdict.reason))
+                continue
+            if self._start(ticket, verdict.pages) and verdict.skipped_head:
+                self.head_skips += 1
+        if self._waiting:
+            logger.info("continuous_admission_blocked request_id=%s reason=slots",
+                        self._waiting[0].request.request_id)
+
+    def _start(self, ticket: Ticket, pages: int) -> bool:
+        request = ticket.request
+        capacity = len(request.input_ids) + request.sampling.max_new_tokens
+        try:
+            self._serial += 1
+            seq = self.runner.open((request.request_id, self._serial), capacity)
+        except Exception as error:
+            ticket.future.set_exception(error)
+            return False
+        self._active.append(Active(
+            ticket=ticket, seq=seq, reserved_pages=pages,
+            queue_seconds=self._clock() - ticket.arrived, prompt_wait_started=ticket.arrived,
+        ))
+        return True
+
+    # ---- the step -----------------------------------------------------------------------------
+    def _run_step(self) -> None:
+        now = self._clock()
+        decoding = [a for a in self._active if a.pending_token_id is not None]
+        work = [PromptWork(a, a.remaining_prompt, a.prompt_wait_started)
+                for a in self._active if a.pending_token_id is None and a.remaining_prompt > 0]
+        portions: List[Tuple[Active, int]] = []
+        if not hold_prompts(len(decoding), self._max_batch_size, work, now):
+            portions = cut_prompts(work, self._prefill_chunk_size, now)
+        # Decode rows first, then prompt portions; the portions' token budget is not
+        # reduced by the decode rows (/root/reference/src/pylon/engine.py:292-298).
+        entries: List[StepEntry] = []
+        ready: List[Active] = []
+        for item in decoding:
+            entries.append(StepEntry(item.seq, [item.pending_token_id], [0]))
+            ready.append(item)
+        for item, count in portions:
+            chunk = item.request.input_ids[item.prompt_offset: item.prompt_offset + count]
+            finishes = item.prompt_offset + count >= len(item.request.input_ids)
+            entries.append(StepEntry(item.seq, chunk, [count - 1] if finishes else []))
+            if finishes:
+                ready.append(item)
+        if not entries:
+            return
+        self.last_step = ([a.request.request_id for a in decoding],
+                          [(a.request.request_id, c) for a, c in portions])
+        started = self._clock()
+        logits = self.runner.step(entries)
+        self.steps_run += 1
+        for item, count in portions:
+            item.prompt_offset += count
+            item.prompt_wait_started = self._clock()
+        token_ids: List[int] = []
+        if ready:
+            token_ids = self.sampler.sample(
+                logits, [(a.request.sampling, len(a.output_ids)) for a in ready]
+            )
+        elif hasattr(self.runner, "synchronize"):
+            self.runner.synchronize()
+        sampled_at = self._clock()
+        elapsed = sampled_at - started
+        for item in decoding:
+            item.inter_token_seconds.append(elapsed)
+        for item, _count in portions:
+            item.prefill_seconds += elapsed
+        finished = set()
+        for item, token_id in zip(ready, token_ids):
+            if not self._accept(item, int(token_id), sampled_at):
+                finished.add(id(item))
+        self._active = [a for a in self._active if id(a) not in finished]
+
+    def _accept(self, item: Active, token_id: int, sampled_at: float) -> bool:
+        """/root/reference/src/pylon/engine.py:598-618: a stop token ends the request and
+        is not emitted; reaching max_new_tokens ends it with "length"."""
+        if item.first_token_at is None:
+            item.first_token_at = sampled_at
+        if token_id in item.request.stop_ids:
+            self._complete(item, "eos")
+            return False
+        item.output_ids.append(token_id)
+        if len(item.output_ids) == item.request.sampling.max_new_tokens:
+            self._complete(item, "length")
+            return False
+        item.pending_token_id = token_id
+        return True
+
+    def _complete(self, item: Active, reason: str) -> None:
+        self.runner.close(item.seq)
+        arrived = item.ticket.arrived
+        result = GenerationResult(
+            output_ids=item.output_ids, finish_reason=reason, prefill_seconds=item.prefill_seconds,
+            inter_token_seconds=item.inter_token_seconds, queue_seconds=item.queue_seconds,
+            first_token_seconds=None if item.first_token_at is None else item.first_token_at - arrived,
+            elapsed_seconds=self._clock() - arrived,
+        )
+        if not item.ticket.future.done():
+            item.ticket.future.set_result(result)
+
+    def _drop_cancelled_active(self) -> None:
+        kept = []
+        for item in self._active:
+            if item.ticket.future.cancelled():
+                self.runner.close(item.seq)
+            else:
+                kept.append(item)
+        self._active = kept
+
+    def _fail_active(self, error: Exception) -> None:
+        """A step that raised (pages ran short, a kernel refused) fails every running
+        request and frees what they hold; waiting requests stay queued."""
+        for item in self._active:
+            self.runner.close(item.seq)
+            if not item.ticket.future.done():
+                item.ticket.future.set_exception(error)
+        self._active = []
+
+    # ---- validation ---------------------------------------------------------------------------
+    def _validate_request(self, input_ids: List[int], stop_ids: frozenset, sampling: Sampling) -> None:
+        """/root/reference/src/pylon/engine.py:731-759."""
+        spec = self.runner.model.spec
+        if not input_ids:
+            raise ValueError("A request prompt must contain at least one token.")
+        for token_id in (*stop_ids, *input_ids):
+            if isinstance(token_id, bool) or not isinstance(token_id, int) or not 0 <= token_id < spec.vocab_size:
+                raise ValueError(f"Token IDs must be between 0 and {spec.vocab_size - 1:,}.")
+        token_count = len(input_ids) + sampling.max_new_tokens
+        if spec.max_positions and token_count > spec.max_positions:
+            raise ValueError(
+                f"Request needs {token_count:,} cache positions, but the model supports "
+                f"{spec.max_positions:,}."
+            )
+        max_tokens = self.kv_budget_pages * self.page_size
+        if token_count > max_tokens:
+            raise ValueError(
+                f"Request needs {token_count:,} KV-cache tokens, but the profiled limit "
+                f"is {max_tokens:,}."
+            )
+
+    # ---- the background thread ----------------------------------------------------------------
+    def _drive(self) -> None:
+        wait = self._config.batch_wait_ms / 1_000
+        while True:
+            with self._wake:
+                while not self._waiting and not self._active and not self._closed:
+                    self._wake.wait()
+                if self._closed:
+                    return
+                if not self._active and self._max_batch_size > 1 and self._waiting:
+                    # Nothing is running: give more arrivals a moment to join the first
+                    # step (/root/reference/src/pylon/scheduler/queue.py:157-166).
+                    deadline = self._waiting[0].arrived + wait
+                    while (self._waiting and len(self._waiting) < self._max_batch_size
+                           and not self._closed):
+                        remaining = deadline - self._clock()
+                        if remaining <= 0:
+                            break
+                        self._wake.wait(remaining)
+                    if self._closed:
+                        return
+            try:
+                self.tick()
+            except Exception as error:  # noqa: BLE001 - a broken tick fails what runs
+                with self._lock:
+                    self._fail_active(error)
+
+
+def _load_runner(config: PylonConfig):
+    import torch
+
+    from .runner import Runner
+
+    if config.model_path is None:
+        raise ValueError("PylonConfig.model_path (or PYLON_MODEL_PATH) names no model folder.")
+    if not torch.cuda.is_available():
+        raise RuntimeError("A GPU is required.")
+    return Runner.from_config(config)

@@ -58,6 +58,38 @@ class Runner:
         runner.config = config
         return runner
 
+    @classmethod
+    def from_config(cls, config, *, device="cuda:0") -> "Runner":
+        """Load ``config.model_path`` and size the page pool: ``config.num_pages`` if given,
+        else from the device memory that is free once the weights are resident
+        (/root/reference/src/pylon/kv/budget.py:70-113: utilisation limit times total
+        memory, minus what is occupied, minus a headroom share for activations)."""
+        if not torch.cuda.is_available():
+            raise RuntimeError("A GPU is required: the step function has no CPU path.")
+        arch, model_config = load_model_config(config.model_path)
+        model = Model(arch.model_spec(model_config), dtype=resolve_dtype(config.dtype), device=device)
+        load_weights(model, arch, model_config, Path(config.model_path))
+        num_pages = config.num_pages
+        if num_pages is None:
+            from ..cache.manager import bytes_per_token
+
+            per_token = bytes_per_token(model.cache_requirements(), model.dtype)
+            free, total = torch.cuda.mem_get_info(model.device)
+            budget = int(total * config.max_gpu_utilization) - (total - free)
+            budget = int(budget * (1.0 - config.kv_cache_headroom_ratio))
+            num_pages = budget // max(1, config.page_size * per_token)
+            ceiling = -(-model.spec.max_positions // config.page_size) * config.max_batch_size
+            num_pages = min(num_pages, ceiling)
+            if num_pages < 1:
+                raise ValueError("The KV budget must hold at least one attention page.")
+        runner = cls(model, page_size=config.page_size, num_pages=int(num_pages),
+                     max_requests=config.max_batch_size)
+        runner.config = model_config
+        return runner
+
+    def synchronize(self) -> None:
+        torch.cuda.synchronize(self.model.device)
+
     # ---- requests -------------------------------------------------------------------------
     def open(self, request_id: Hashable, capacity: Optional[int] = None) -> Sequence:
         max_positions = self.model.spec.max_positions

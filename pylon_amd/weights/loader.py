@@ -78,6 +78,7 @@ def load_weights(model, arch: Architecture, config, folder) -> None:
     found: Dict[str, Tuple[Path, Tuple[int, ...], str]] = {}
     unexpected: List[str] = []
     wrong: List[str] = []
+    present = set()
     for path in files:
         with safe_open(str(path), framework="pt", device="cpu") as f:
             for name in f.keys():
@@ -87,6 +88,7 @@ def load_weights(model, arch: Architecture, config, folder) -> None:
                 if target is None:
                     unexpected.append(name)
                     continue
+                present.add(name)
                 if target.param not in params:
                     wrong.append(f"{name}: the model has no parameter {target.param}")
                     continue
@@ -98,7 +100,7 @@ def load_weights(model, arch: Architecture, config, folder) -> None:
                     wrong.append(f"{name}: stored as {stored}, which a {target.role} cannot be")
                     continue
                 found[name] = (path, shape, stored)
-    missing = [n for n, t in targets.items() if n not in found and not t.optional]
+    missing = [n for n, t in targets.items() if n not in present and not t.optional]
     if missing or unexpected or wrong:
         raise WeightsError(missing, unexpected, wrong)
 
