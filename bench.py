@@ -1,0 +1,217 @@
+"""Decode and prefill throughput of the engine at the Qwen3-4B shape, with random weights
+and uniform-random token ids, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+
+A "step" is one decode step: one token for each of ``batch`` running requests through
+the step function, then greedy sampling on the device and the copy of the chosen ids to
+the host.  ``value`` is decoded tokens per second at the default batch of 8.  The same
+line carries the prefill of 2,048 tokens, the decode step's share of the HBM roofline,
+and decode rates at batch 1 and 64.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+# MI355X published peaks.
+HBM_BYTES_PER_S = 8.0e12
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+# The benchmark configuration: Qwen3-4B shape.
+SHAPE_4B = dict(
+    num_hidden_layers=36, hidden_size=2560, num_attention_heads=32, num_key_value_heads=8,
+    head_dim=128, intermediate_size=9728, vocab_size=151936, rope_theta=5000000.0,
+    rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=8192,
+)
+CONTEXT_LENGTH = 8192
+PAGE_SIZE = 256
+PROMPT_LEN = 128
+NEW_TOKENS = 512
+PREFILL_TOKENS = 2048
+
+
+def config_json(layers: int) -> dict:
+    cfg = dict(SHAPE_4B, num_hidden_layers=layers)
+    cfg.update(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_act="silu")
+    return cfg
+
+
+def build_runner(layers: int, dtype: str, max_requests: int, num_pages: int, graphs: bool):
+    import torch
+
+    from pylon_amd.config import resolve
+    from pylon_amd.engine import Model, Runner, resolve_dtype
+
+    raw = config_json(layers)
+    arch = resolve(raw)
+    cfg = arch.parse_config(raw)
+    model = Model(arch.model_spec(cfg), dtype=resolve_dtype(dtype), device="cuda:0")
+    model.init_random(seed=0)
+    runner = Runner(model, page_size=PAGE_SIZE, num_pages=num_pages, max_requests=max_requests)
+    if graphs and hasattr(runner, "enable_graphs"):
+        runner.enable_graphs()
+    torch.cuda.synchronize()
+    return runner, cfg
+
+
+def weight_bytes(runner) -> int:
+    """Bytes of every weight a decode step reads once: all layer matrices and vectors and
+    the vocabulary head (the embedding table itself is only gathered from)."""
+    total = 0
+    for path, owner, name in runner.model.named_params():
+        if path == "embed" and not runner.model.spec.tie_word_embeddings:
+            continue
+        t = owner.params[name]
+        total += t.numel() * t.element_size()
+    return total
+
+
+def linear_flops_per_token(cfg) -> float:
+    q = cfg.num_attention_heads * cfg.head_dim
+    kv = cfg.num_key_value_heads * cfg.head_dim
+    per_layer = cfg.hidden_size * (q + 2 * kv) + q * cfg.hidden_size + 3 * cfg.hidden_size * cfg.intermediate_size
+    return 2.0 * cfg.num_hidden_layers * per_layer
+
+
+def decode_run(runner, cfg, batch: int, steps: int, warmup: int, seed: int):
+    """Prefill ``batch`` prompts of PROMPT_LEN random ids, then time ``steps`` decode steps."""
+    import numpy as np
+    import torch
+
+    from pylon_amd.engine import StepEntry
+    from pylon_amd.kernels import ops
+
+    rng = np.random.default_rng(seed)
+    seqs = [runner.open(f"b{batch}-{i}") for i in range(batch)]
+    prompts = [rng.integers(0, cfg.vocab_size, PROMPT_LEN).tolist() for _ in range(batch)]
+    # prompts in portions of up to 2048 tokens, as the scheduler would cut them
+    per_step = max(1, PREFILL_TOKENS // PROMPT_LEN)
+    logits = []
+    for lo in range(0, batch, per_step):
+        part = list(range(lo, min(batch, lo + per_step)))
+        out = runner.step([StepEntry(seqs[i], prompts[i], [PROMPT_LEN - 1]) for i in part])
+        logits.append(out)
+    tokens = ops.argmax(torch.cat(logits)).cpu().tolist()
+
+    def one_step(tokens):
+        out = runner.step([StepEntry(seqs[i], [tokens[i]], [0]) for i in range(batch)])
+        return ops.argmax(out).cpu().tolist()
+
+    for _ in range(warmup):
+        tokens = one_step(tokens)
+    torch.cuda.synchronize()
+    context_sum = 0
+    started = time.perf_counter()
+    for _ in range(steps):
+        context_sum += sum(s.length + 1 for s in seqs)
+        tokens = one_step(tokens)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - started
+    for s in seqs:
+        runner.close(s)
+    return elapsed, context_sum / steps  # seconds, mean cached tokens read per step (all rows)
+
+
+def prefill_run(runner, cfg, repeats: int, seed: int):
+    """One prompt of PREFILL_TOKENS random ids in one step; the median of ``repeats`` runs."""
+    import numpy as np
+    import torch
+
+    from pylon_amd.engine import StepEntry
+
+    rng = np.random.default_rng(seed)
+    times = []
+    for r in range(repeats + 1):
+        seq = runner.open(f"prefill-{r}")
+        prompt = rng.integers(0, cfg.vocab_size, PREFILL_TOKENS).tolist()
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        out = runner.step([StepEntry(seq, prompt, [PREFILL_TOKENS - 1])])
+        out.cpu()
+        times.append(time.perf_counter() - started)
+        runner.close(seq)
+    times = sorted(times[1:])  # the first run warms the library's kernels up
+    return times[len(times) // 2]
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=NEW_TOKENS)
+    parser.add_argument("--warmup", type=int, default=16)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--layers", type=int, default=SHAPE_4B["num_hidden_layers"])
+    parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
+    parser.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
+    parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    parser.add_argument("--no-prefill", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this engine runs on one GPU; --gpus must be 1")
+        return 2
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: A GPU is required.", file=sys.stderr)
+        return 1
+
+    max_batch = max(64, args.batch)
+    pages_per_request = CONTEXT_LENGTH // PAGE_SIZE
+    runner, cfg = build_runner(args.layers, args.dtype, max_requests=max_batch,
+                               num_pages=max_batch * pages_per_request, graphs=not args.no_graphs)
+    dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
+    steps = min(args.steps, CONTEXT_LENGTH - PROMPT_LEN - args.warmup)
+
+    elapsed, mean_context = decode_run(runner, cfg, args.batch, steps, args.warmup, seed=1)
+    ms_per_step = 1e3 * elapsed / steps
+    value = args.batch * steps / elapsed
+    per_token = runner.manager.bytes_per_token
+    step_bytes = weight_bytes(runner) + mean_context * per_token
+    achieved = step_bytes / (elapsed / steps)
+
+    record = {
+        "metric": "decode tokens/s, Qwen3-4B shape, batch 8, 128-token prompts",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": dtype_key, "data": "synthetic",
+        "config": {
+            "model": "qwen3-4b-shape-random", "layers": args.layers,
+            "layers_full": SHAPE_4B["num_hidden_layers"], "hidden": cfg.hidden_size,
+            "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+            "global_batch": args.batch, "seq_len": PROMPT_LEN, "new_tokens": steps,
+            "context_length": CONTEXT_LENGTH, "page_size": PAGE_SIZE, "prefill_tokens": PREFILL_TOKENS,
+            "hip_graphs": bool(getattr(runner, "graphs", None)), "parallelism": "single-gpu",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_BYTES_PER_S / 1e9,
+                     "unit": "GB/s", "frac": round(achieved / HBM_BYTES_PER_S, 4)},
+    }
+    if not args.no_prefill:
+        seconds = prefill_run(runner, cfg, repeats=5, seed=2)
+        attention = 4.0 * cfg.num_hidden_layers * cfg.num_attention_heads * cfg.head_dim * (
+            PREFILL_TOKENS * (PREFILL_TOKENS + 1) / 2)
+        flops = linear_flops_per_token(cfg) * PREFILL_TOKENS + attention + 2.0 * cfg.hidden_size * cfg.vocab_size
+        record["prefill"] = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
+                             "ms": round(1e3 * seconds, 3),
+                             "frac": round(flops / seconds / PEAK_FLOPS[dtype_key], 4)}
+    if not args.no_points:
+        points = {}
+        for batch in (1, 64):
+            n = min(steps, 256)
+            e, _ = decode_run(runner, cfg, batch, n, args.warmup, seed=3 + batch)
+            points[f"decode_b{batch}"] = round(batch * n / e, 1)
+        record["points"] = points
+    print(json.dumps(record))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

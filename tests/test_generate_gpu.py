@@ -1,0 +1,149 @@
+"""Generation through the entry point against the plain implementation: greedy, seeded
+temperature sampling, the first tokens of a sequence, and long decoding."""
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import CONFIGS, make_model_folder, random_tokens, read_folder
+from tests.plain import qwen3 as plain
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tmp(tmp_path_factory):
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    return tmp_path_factory.mktemp("gen")
+
+
+def plain_generate(weights, cfg, prompt, count, pick):
+    tokens = list(prompt)
+    out = []
+    for i in range(count):
+        nxt = pick(plain.forward(weights, cfg, tokens)[-1], i)
+        out.append(nxt)
+        tokens.append(nxt)
+    return out
+
+
+def margins_ok(weights, cfg, prompt, produced, floor):
+    """True if every greedy choice of the plain model wins by more than ``floor``."""
+    tokens = list(prompt)
+    for tok in produced:
+        row = np.sort(plain.forward(weights, cfg, tokens)[-1])
+        if row[-1] - row[-2] <= floor:
+            return False
+        tokens.append(tok)
+    return True
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_engine(tmp, dtype):
+    """Tiny A's workload: prompts of 5, 17 and 33 tokens, 16 greedy tokens each, all three
+    running together through the scheduler with prompts cut into portions of 8."""
+    from pylon_amd.engine.engine import Engine
+    from pylon_amd.sampling import Sampling
+
+    folder = make_model_folder(tmp, "A", dtype=dtype, std=0.08)
+    cfg, weights = read_folder(folder)
+    prompts = [random_tokens(cfg["vocab_size"], n, 70 + n) for n in (5, 17, 33)]
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=12, max_batch_size=4,
+                                prefill_chunk_size=8)
+    try:
+        results = engine.generate(prompts, Sampling(max_new_tokens=16, temperature=0.0))
+    finally:
+        engine.close()
+    assert engine.runner.manager.free_pages == 12
+    for prompt, result in zip(prompts, results):
+        want = plain_generate(weights, cfg, prompt, 16, lambda row, i: plain.greedy(row))
+        assert result.finish_reason == "length" and len(result.output_ids) == 16
+        if dtype == "float32":
+            assert result.output_ids == want
+        else:
+            # bfloat16 may flip a near-tie; up to the first flip the tokens must agree,
+            # and a flip is only allowed where the plain model's margin is small
+            agree = next((i for i, (a, b) in enumerate(zip(result.output_ids, want)) if a != b), 16)
+            assert agree == 16 or not margins_ok(weights, cfg, prompt, want[: agree + 1], 0.02)
+
+
+def test_stop_token_and_first_token_from_a_one_token_prompt(tmp):
+    from pylon_amd.engine.engine import Engine
+    from pylon_amd.sampling import Sampling
+
+    folder = make_model_folder(tmp, "B", dtype="float32", std=0.08)
+    cfg, weights = read_folder(folder)
+    prompt = [7]
+    want = plain_generate(weights, cfg, prompt, 8, lambda row, i: plain.greedy(row))
+    engine = Engine.from_folder(folder, dtype="float32", page_size=32, num_pages=4)
+    try:
+        got = engine.generate([prompt], Sampling(max_new_tokens=8, temperature=0.0))[0]
+        assert got.output_ids == want
+        stop = want[3]
+        first = want.index(stop)
+        cut = engine.generate([prompt], Sampling(max_new_tokens=8, temperature=0.0), eos_token_id=stop)[0]
+        assert cut.finish_reason == "eos" and cut.output_ids == want[:first]
+    finally:
+        engine.close()
+
+
+def test_seeded_temperature_sampling_matches_the_plain_rule(tmp):
+    """Tiny B's workload: prompts of 1, 31, 64 and 100 tokens in portions of 48 beside
+    decodes, temperature 0.8 from a fixed seed, 24 tokens each.  The engine's draw for
+    token i of a request is the cumulative distribution read at uniform(seed, i)."""
+    from pylon_amd.engine.engine import Engine
+    from pylon_amd.sampling import Sampling, uniform
+
+    folder = make_model_folder(tmp, "B", dtype="float32", std=0.08)
+    cfg, weights = read_folder(folder)
+    prompts = [random_tokens(cfg["vocab_size"], n, 90 + n) for n in (1, 31, 64, 100)]
+    for top_p in (1.0, 0.9):
+        sampling = Sampling(max_new_tokens=24, temperature=0.8, top_p=top_p, seed=1234)
+        engine = Engine.from_folder(folder, dtype="float32", page_size=32, num_pages=16,
+                                    max_batch_size=4, prefill_chunk_size=48)
+        try:
+            results = engine.generate(prompts, sampling)
+            alone = engine.generate([prompts[2]], sampling)[0]
+        finally:
+            engine.close()
+        # a request's tokens do not depend on what ran beside it
+        assert alone.output_ids == results[2].output_ids
+        for prompt, result in zip(prompts, results):
+            tokens = list(prompt)
+            for i, tok in enumerate(result.output_ids):
+                row = plain.forward(weights, cfg, tokens)[-1]
+                u = uniform(1234, i)
+                want = plain.sample_with_uniform(row, 0.8, top_p, u)
+                if tok != want:
+                    p = plain.sampling_distribution(row, 0.8, top_p)
+                    cdf = np.cumsum(p)
+                    assert p[tok] > 0 and abs(cdf[min(tok, want)] - u) < 1e-4, (i, tok, want)
+                tokens.append(tok)
+        assert len({tuple(r.output_ids) for r in results}) == 4
+
+
+def test_long_decoding_stays_on_the_plain_model(tmp):
+    """600 tokens decoded one by one after a short prompt (crossing many pages), with the
+    logits of the engine's own token sequence compared at the end."""
+    from pylon_amd.engine import Runner, StepEntry
+
+    folder = make_model_folder(tmp, "C", dtype="float32", std=0.08)
+    cfg, weights = read_folder(folder)
+    prompt = random_tokens(cfg["vocab_size"], 11, 3)
+    runner = Runner.from_folder(folder, dtype="float32", page_size=64, num_pages=10, max_requests=2)
+    seq = runner.open("long")
+    logits = runner.step([StepEntry(seq, prompt, [len(prompt) - 1])])
+    tokens, rows = list(prompt), []
+    for _ in range(600):
+        rows.append(logits[0].cpu().numpy())
+        nxt = int(torch.argmax(logits[0]).item())
+        tokens.append(nxt)
+        logits = runner.step([StepEntry(seq, [nxt], [0])])
+    assert seq.length == 611 and len(seq.pages[0]) == 10
+    want = plain.forward(weights, cfg, tokens[:-1])[len(prompt) - 1:]
+    got = np.stack(rows)
+    err = np.abs(got - want).max(axis=1)
+    assert err.max() <= 2e-5 * np.abs(want).max(), int(err.argmax())
+    assert len(set(tokens[len(prompt):])) > 3  # the model does not just repeat one token

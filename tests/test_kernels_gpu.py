@@ -1,0 +1,326 @@
+"""Each kernel alone against a plain float64 reference of the same operation, at sizes
+other than the engine's (odd widths, head sizes in steps of 16, vocabularies that are no
+power of two), in float32 and in bfloat16."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from pylon_amd.kernels import check_device, ops as _ops
+
+    check_device()
+    return _ops
+
+
+def rnd(shape, seed, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def tol(dtype, scale=1.0):
+    # float32: a few ulps of accumulated rounding; bfloat16: one rounding of the result
+    # (2^-9 relative) plus rounding of inputs that both sides share.
+    return (2e-6 if dtype == torch.float32 else 6e-3) * scale
+
+
+def f64(t):
+    return t.detach().cpu().to(torch.float64).numpy()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(ops, dtype):
+    table = rnd((301, 72), 1, dtype)
+    ids = torch.tensor([0, 300, 17, 17, 5], dtype=torch.int32)
+    out = ops.embed(ids.to(DEV), table.to(DEV), scale=0.5)
+    assert out.dtype == torch.float32
+    assert np.array_equal(f64(out), f64(table)[ids.numpy()] * 0.5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dim", [80, 1000, 2560 + 16])
+def test_rmsnorm_and_fused_residual(ops, dtype, dim):
+    eps = 3e-5
+    x = rnd((7, dim), 2, torch.float32, 2.0)
+    delta = rnd((7, dim), 3, dtype)
+    w = 1 + 0.3 * rnd((dim,), 4)
+
+    def ref(v):
+        return v / np.sqrt((v * v).mean(-1, keepdims=True) + eps) * f64(w)
+
+    got = ops.rmsnorm(x.to(dtype).to(DEV), w.to(DEV), eps, out_dtype=dtype)
+    want = ref(f64(x.to(dtype)))
+    assert np.abs(f64(got) - want).max() <= tol(dtype, np.abs(want).max())
+    # fused: resid += delta (float32), out = norm(resid)
+    resid = x.clone().to(DEV)
+    got = ops.add_rmsnorm(resid, delta.to(DEV), w.to(DEV), eps, dtype)
+    summed = f64(x) + f64(delta)
+    assert np.abs(f64(resid) - summed).max() <= 1e-6 * np.abs(summed).max()
+    assert np.abs(f64(got) - ref(summed)).max() <= tol(dtype, np.abs(ref(summed)).max())
+    # with picked rows the residual stays as it was
+    resid = x.clone().to(DEV)
+    idx = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    got = ops.add_rmsnorm(resid, delta.to(DEV), w.to(DEV), eps, dtype, row_idx=idx)
+    assert torch.equal(resid.cpu(), x)
+    assert np.abs(f64(got) - ref(summed)[[6, 0, 3]]).max() <= tol(dtype, np.abs(ref(summed)).max())
+    # no delta: plain norm of the residual
+    got = ops.add_rmsnorm(resid, None, w.to(DEV), eps, dtype)
+    assert np.abs(f64(got) - ref(f64(x))).max() <= tol(dtype, np.abs(ref(f64(x))).max())
+    r2 = x.clone().to(DEV)
+    ops.residual_add(r2, delta.to(DEV))
+    assert np.abs(f64(r2) - summed).max() <= 1e-6 * np.abs(summed).max()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_gate(ops, dtype):
+    gu = rnd((5, 2 * 176), 5, dtype, 3.0)
+    got = ops.silu_gate(gu.to(DEV))
+    g, u = f64(gu)[:, :176], f64(gu)[:, 176:]
+    want = g / (1 + np.exp(-g)) * u
+    assert np.abs(f64(got) - want).max() <= tol(dtype, np.abs(want).max())
+    zero_gate = gu.clone()
+    zero_gate[:, :176] = 0
+    assert float(ops.silu_gate(zero_gate.to(DEV)).abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("combo", [
+    (torch.float32, torch.float32, torch.float32),
+    (torch.bfloat16, torch.bfloat16, torch.bfloat16),
+    (torch.bfloat16, torch.bfloat16, torch.float32),
+    (torch.bfloat16, torch.float32, torch.bfloat16),
+])
+@pytest.mark.parametrize("shape", [(1, 96, 80), (5, 301, 176), (67, 130, 1000), (130, 64, 64)])
+def test_gemm_tiled(ops, combo, shape):
+    a_dt, w_dt, o_dt = combo
+    m, n, k = shape
+    a, w = rnd((m, k), 6, a_dt), rnd((n, k), 7, w_dt, 0.1)
+    got = ops.gemm_tiled(a.to(DEV), w.to(DEV), out_dtype=o_dt)
+    want = f64(a) @ f64(w).T
+    assert got.dtype == o_dt
+    assert np.abs(f64(got) - want).max() <= tol(o_dt, np.abs(want).max())
+
+
+def test_gemm_rows_do_not_depend_on_the_batch(ops):
+    # float32: bit-identical whatever rows share the launch
+    a, w = rnd((70, 200), 8), rnd((90, 200), 9)
+    whole = ops.gemm_tiled(a.to(DEV), w.to(DEV))
+    for lo, hi in ((0, 1), (3, 4), (63, 70), (10, 40)):
+        part = ops.gemm_tiled(a[lo:hi].contiguous().to(DEV), w.to(DEV))
+        assert torch.equal(part, whole[lo:hi])
+
+
+def plain_rope(x, pos, inv_freq, rot):
+    # x: [..., d]; rotate the first `rot` elements, pairing i with i + rot/2
+    ang = (np.float32(pos) * inv_freq.astype(np.float32)).astype(np.float64)
+    c, s = np.cos(ang), np.sin(ang)
+    out = x.copy()
+    a, b = x[..., : rot // 2], x[..., rot // 2: rot]
+    out[..., : rot // 2] = a * c - b * s
+    out[..., rot // 2: rot] = b * c + a * s
+    return out
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("geom", [(5, 5, 48, 48), (6, 2, 16, 16), (3, 1, 128, 64), (2, 2, 80, 0)])
+def test_qkv_prepare(ops, dtype, geom):
+    nh, nkv, hd, rot = geom
+    tokens, page, pages, eps = 9, 4, 6, 2e-5
+    qkv = rnd((tokens, (nh + 2 * nkv) * hd), 10, dtype)
+    qw, kw = 1 + 0.2 * rnd((hd,), 11), 1 + 0.2 * rnd((hd,), 12)
+    inv_freq = (1.0 / (1000.0 ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))) if rot else None
+    positions = torch.tensor([0, 1, 2, 3, 40, 41, 7, 1000, 5], dtype=torch.int32)
+    slots = torch.tensor([4, 5, 6, 7, 0, 1, 23, 12, -1], dtype=torch.int32)
+    kc = torch.zeros((pages, page, nkv, hd), dtype=dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    q = torch.empty((tokens, nh, hd), dtype=dtype, device=DEV)
+    ops.qkv_prepare(qkv.to(DEV), q, kc, vc, n_heads=nh, n_kv_heads=nkv, head_dim=hd,
+                    q_weight=qw.to(DEV), k_weight=kw.to(DEV), eps=eps,
+                    inv_freq=inv_freq.to(DEV) if rot else None, rot_dim=rot,
+                    positions=positions.to(DEV), slot_map=slots.to(DEV), store_kv=True)
+    raw = f64(qkv).reshape(tokens, nh + 2 * nkv, hd)
+
+    def norm(v, w):
+        return v / np.sqrt((v * v).mean(-1, keepdims=True) + eps) * f64(w)
+
+    kflat, vflat = f64(kc).reshape(pages * page, nkv, hd), f64(vc).reshape(pages * page, nkv, hd)
+    for t in range(tokens):
+        qn, kn = norm(raw[t, :nh], qw), norm(raw[t, nh:nh + nkv], kw)
+        if rot:
+            qn = plain_rope(qn, int(positions[t]), inv_freq.numpy(), rot)
+            kn = plain_rope(kn, int(positions[t]), inv_freq.numpy(), rot)
+        assert np.abs(f64(q)[t] - qn).max() <= tol(dtype, np.abs(qn).max())
+        if slots[t] >= 0:
+            assert np.abs(kflat[slots[t]] - kn).max() <= tol(dtype, np.abs(kn).max())
+            assert np.array_equal(vflat[slots[t]], raw[t, nh + nkv:])  # v: neither normed nor rotated
+    untouched = sorted(set(range(pages * page)) - {int(s) for s in slots if s >= 0})
+    assert np.abs(kflat[untouched]).max() == 0 and np.abs(vflat[untouched]).max() == 0
+    # without norm weights and without storing: q only, rotated only
+    q2 = torch.empty_like(q)
+    ops.qkv_prepare(qkv[:, : nh * hd].contiguous().to(DEV), q2, None, None, n_heads=nh, n_kv_heads=nkv,
+                    head_dim=hd, q_weight=None, k_weight=None, eps=eps,
+                    inv_freq=inv_freq.to(DEV) if rot else None, rot_dim=rot,
+                    positions=positions.to(DEV), slot_map=None, store_kv=False)
+    for t in range(tokens):
+        want = plain_rope(raw[t, :nh], int(positions[t]), inv_freq.numpy(), rot) if rot else raw[t, :nh]
+        assert np.abs(f64(q2)[t] - want).max() <= tol(dtype, np.abs(want).max())
+
+
+def plain_attention(q, keys, values, scale, window):
+    """q: [heads, d] at the last position of keys [kv, n, d]."""
+    heads = q.shape[0]
+    group = heads // keys.shape[0]
+    n = keys.shape[1]
+    lo = max(0, n - window) if window else 0
+    out = np.zeros_like(q)
+    for h in range(heads):
+        k, v = keys[h // group, lo:], values[h // group, lo:]
+        s = k @ q[h] * scale
+        p = np.exp(s - s.max())
+        out[h] = (p / p.sum()) @ v
+    return out
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("geom", [(4, 2, 16, 16, None), (6, 1, 32, 32, None), (5, 5, 48, 16, 70),
+                                  (8, 2, 128, 64, None), (2, 1, 256, 16, 33)])
+def test_paged_attention(ops, dtype, geom):
+    nh, nkv, hd, page, window = geom
+    lengths = [1, 65, 130, 2 * page, 2 * page + 1]  # tokens already cached per request (incl. the queries)
+    n_pages = sum(-(-n // page) for n in lengths) + 3
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(13)).tolist()
+    width = max(-(-n // page) for n in lengths)
+    table = torch.zeros((len(lengths), width), dtype=torch.int32)
+    kc = rnd((n_pages, page, nkv, hd), 14, dtype)
+    vc = rnd((n_pages, page, nkv, hd), 15, dtype)
+    cursor = 0
+    for r, n in enumerate(lengths):
+        for i in range(-(-n // page)):
+            table[r, i] = perm[cursor]
+            cursor += 1
+    # queries: the last min(3, n) positions of every request, packed
+    tok_row, positions = [], []
+    for r, n in enumerate(lengths):
+        for p in range(max(0, n - 3), n):
+            tok_row.append(r)
+            positions.append(p)
+    q = rnd((len(tok_row), nh, hd), 16, dtype)
+    scale = 1 / math.sqrt(hd)
+    got = ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV),
+                              torch.tensor(tok_row, dtype=torch.int32, device=DEV),
+                              torch.tensor(positions, dtype=torch.int32, device=DEV),
+                              page_size=page, window=window, scale=scale)
+    kf, vf = f64(kc), f64(vc)
+    for i, (r, p) in enumerate(zip(tok_row, positions)):
+        idx = [(int(table[r, j // page]), j % page) for j in range(p + 1)]
+        keys = np.stack([kf[a, b] for a, b in idx], axis=1)  # [kv, n, d]
+        vals = np.stack([vf[a, b] for a, b in idx], axis=1)
+        want = plain_attention(f64(q)[i], keys, vals, scale, window)
+        assert np.abs(f64(got)[i] - want).max() <= tol(dtype, max(1.0, np.abs(want).max())), (i, r, p)
+
+
+def test_attention_finds_one_far_key_among_hundreds(ops):
+    # Random keys would hide a key that is skipped; here one far key matches the query
+    # exactly and strongly, so the output must be (almost) that key's value.
+    nh, nkv, hd, page = 2, 1, 64, 16
+    n = 777
+    for far in (0, 15, 16, 400, 776 - 64, 776):
+        kc = rnd((50, page, nkv, hd), 17) * 0.01
+        vc = rnd((50, page, nkv, hd), 18)
+        table = torch.arange(49, -1, -1, dtype=torch.int32).reshape(1, 50)
+        q = rnd((1, nh, hd), 19)
+        page_id, off = int(table[0, far // page]), far % page
+        kc[page_id, off, 0] = q[0, 0] * 4.0
+        got = ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV),
+                                  torch.zeros(1, dtype=torch.int32, device=DEV),
+                                  torch.tensor([n - 1], dtype=torch.int32, device=DEV),
+                                  page_size=page, window=None, scale=1.0)
+        assert torch.allclose(got[0, 0].cpu(), vc[page_id, off, 0], atol=1e-3), far
+
+
+def test_attention_window_edge(ops):
+    # the key at distance `window` must be invisible, the one at distance window-1 visible
+    nh, nkv, hd, page, window = 1, 1, 16, 16, 37
+    kc = torch.zeros((8, page, nkv, hd))
+    vc = rnd((8, page, nkv, hd), 20)
+    table = torch.arange(8, dtype=torch.int32).reshape(1, 8)
+    q = torch.ones((1, nh, hd))
+    pos = 100
+    for key, visible in ((pos - window, False), (pos - window + 1, True)):
+        k2 = kc.clone()
+        k2[key // page, key % page, 0] = 8.0  # a key that would dominate
+        got = ops.paged_attention(q.to(DEV), k2.to(DEV), vc.to(DEV), table.to(DEV),
+                                  torch.zeros(1, dtype=torch.int32, device=DEV),
+                                  torch.tensor([pos], dtype=torch.int32, device=DEV),
+                                  page_size=page, window=window, scale=1.0)
+        hit = torch.allclose(got[0, 0].cpu(), vc[key // page, key % page, 0], atol=1e-3)
+        assert hit == visible, key
+
+
+def test_sampling_kernels(ops):
+    from tests.plain import qwen3 as plain
+
+    vocab = 1237
+    logits = rnd((6, vocab), 21, scale=3.0)
+    logits[2, 55] = logits[2, 900] = logits[2].max() + 1  # a tie: the lowest index wins
+    dev = logits.to(DEV)
+    assert ops.argmax(dev).cpu().tolist() == [int(np.argmax(f64(logits)[r])) for r in range(6)]
+    assert ops.argmax(dev).cpu().tolist()[2] == 55
+    temps = torch.tensor([0.0, 0.7, 1.0, 1.3, 0.5, 2.0])
+    tops = torch.tensor([1.0, 1.0, 0.9, 0.5, 0.05, 0.95])
+    for trial in range(12):
+        u = torch.rand(6, generator=torch.Generator().manual_seed(100 + trial))
+        got = ops.sample(dev, temps.to(DEV), tops.to(DEV), u.to(DEV)).cpu().tolist()
+        for r in range(6):
+            p = plain.sampling_distribution(f64(logits)[r], float(temps[r]), float(tops[r])) if temps[r] > 0 else None
+            want = plain.sample_with_uniform(f64(logits)[r], float(temps[r]), float(tops[r]), float(u[r]))
+            if got[r] != want:
+                # float32 sums may land on the other side of a boundary of the cumulative
+                # distribution; then the draw must be an adjacent kept token and u must
+                # lie within rounding of that boundary.
+                cdf = np.cumsum(p)
+                assert p[got[r]] > 0 and abs(cdf[min(got[r], want)] - float(u[r])) < 1e-5, (trial, r)
+    # top-p keeps exactly the tokens the plain rule keeps: with u just below 1 the draw is
+    # the last kept token in vocabulary order
+    almost_one = torch.full((6,), 1.0 - 2 ** -24)
+    got = ops.sample(dev, temps.to(DEV), tops.to(DEV), almost_one.to(DEV)).cpu().tolist()
+    for r in range(1, 6):
+        p = plain.sampling_distribution(f64(logits)[r], float(temps[r]), float(tops[r]))
+        assert got[r] == int(np.nonzero(p)[0][-1]), r
+    # empirical frequencies match softmax on a small distribution
+    small = torch.log(torch.tensor([[0.5, 0.25, 0.125, 0.125]])).repeat(4000, 1).to(DEV)
+    us = torch.rand(4000, generator=torch.Generator().manual_seed(3)).to(DEV)
+    draws = ops.sample(small, torch.ones(4000, device=DEV), torch.ones(4000, device=DEV), us).cpu().numpy()
+    freq = np.bincount(draws, minlength=4) / 4000
+    assert np.abs(freq - [0.5, 0.25, 0.125, 0.125]).max() < 0.03
+
+
+def test_kernels_refuse_what_they_cannot_do(ops):
+    from pylon_amd.kernels import KernelError
+
+    q = torch.zeros((1, 2, 24), device=DEV)
+    kc = torch.zeros((2, 16, 1, 24), device=DEV)
+    z = torch.zeros(1, dtype=torch.int32, device=DEV)
+    with pytest.raises(KernelError, match="multiple of 16"):
+        ops.paged_attention(q, kc, kc, torch.zeros((1, 1), dtype=torch.int32, device=DEV), z, z,
+                            page_size=16, window=None, scale=1.0)
+    with pytest.raises(KernelError, match="cannot be grouped"):
+        ops.paged_attention(torch.zeros((1, 3, 32), device=DEV), torch.zeros((2, 16, 2, 32), device=DEV),
+                            torch.zeros((2, 16, 2, 32), device=DEV),
+                            torch.zeros((1, 1), dtype=torch.int32, device=DEV), z, z,
+                            page_size=16, window=None, scale=1.0)
+    with pytest.raises(KernelError, match="no CPU path"):
+        ops.rmsnorm(torch.zeros((2, 8)), torch.ones(8), 1e-6)
+    with pytest.raises(KernelError, match="float32 and bfloat16"):
+        ops.rmsnorm(torch.zeros((2, 8), dtype=torch.float16, device=DEV), torch.ones(8, device=DEV), 1e-6)
+    with pytest.raises(KernelError, match="cannot multiply"):
+        ops.gemm_tiled(torch.zeros((2, 8), device=DEV), torch.zeros((4, 9), device=DEV))
