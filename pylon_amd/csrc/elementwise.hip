@@ -40,6 +40,7 @@ extern "C" int pylon_embed(float* out, const void* table, int table_dtype, const
 // stores that sum back into resid (only meaningful without row_idx).
 template <typename TX, typename TD, typename TO>
 __global__ void rmsnorm_kernel(TO* __restrict__ out, TX* x, const TD* __restrict__ delta,
+                               int n_delta, long long delta_stride,
                                const float* __restrict__ w, const int* __restrict__ row_idx,
                                int dim, float eps, int write_resid) {
   __shared__ float scratch[16];
@@ -56,7 +57,10 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, TX* x, const TD* __restrict
   for (int i = threadIdx.x; i < dim; i += blockDim.x, ++n) {
     float v = to_float(xr[i]);
     if (dr) {
-      v += to_float(dr[i]);
+      // partial sums of the previous matrix product are added in a fixed order
+      float d = to_float(dr[i]);
+      for (int p = 1; p < n_delta; ++p) d += to_float(dr[i + p * delta_stride]);
+      v += d;
       if (write_resid) xr[i] = from_float<TX>(v);
     }
     if (n < KEEP) held[n] = v;
@@ -71,23 +75,27 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, TX* x, const TD* __restrict
       v = held[n];
     } else {
       v = to_float(xr[i]);
-      if (dr && !write_resid) v += to_float(dr[i]);
+      if (dr && !write_resid) {
+        float d = to_float(dr[i]);
+        for (int p = 1; p < n_delta; ++p) d += to_float(dr[i + p * delta_stride]);
+        v += d;
+      }
     }
     yr[i] = from_float<TO>((v * inv) * w[i]);
   }
 }
 
 template <typename TX, typename TD>
-static void launch_rmsnorm_out(void* out, int out_dtype, TX* x, const TD* delta, const float* w,
-                               const int* row_idx, int rows, int dim, float eps, int write_resid,
-                               hipStream_t stream) {
-  dim3 grid(rows), block(256);
+static void launch_rmsnorm_out(void* out, int out_dtype, TX* x, const TD* delta, int n_delta,
+                               long long delta_stride, const float* w, const int* row_idx, int rows,
+                               int dim, float eps, int write_resid, hipStream_t stream) {
+  dim3 grid(rows), block(dim >= 2048 ? 512 : 256);
   if (out_dtype == PYLON_F32)
     hipLaunchKernelGGL((rmsnorm_kernel<TX, TD, float>), grid, block, 0, stream, (float*)out, x, delta,
-                       w, row_idx, dim, eps, write_resid);
+                       n_delta, delta_stride, w, row_idx, dim, eps, write_resid);
   else
     hipLaunchKernelGGL((rmsnorm_kernel<TX, TD, bf16_t>), grid, block, 0, stream, (bf16_t*)out, x,
-                       delta, w, row_idx, dim, eps, write_resid);
+                       delta, n_delta, delta_stride, w, row_idx, dim, eps, write_resid);
 }
 
 // out[r] = rmsnorm(x[idx(r)]) for any input dtype.
@@ -98,30 +106,32 @@ extern "C" int pylon_rmsnorm(void* out, int out_dtype, const void* x, int x_dtyp
   PYLON_REQUIRE(eps >= 0.f, "rmsnorm: eps must not be negative");
   if (rows == 0) return 0;
   if (x_dtype == PYLON_F32)
-    launch_rmsnorm_out<float, float>(out, out_dtype, (float*)x, nullptr, w, row_idx, rows, dim, eps, 0,
-                                     stream);
+    launch_rmsnorm_out<float, float>(out, out_dtype, (float*)x, nullptr, 0, 0, w, row_idx, rows, dim,
+                                     eps, 0, stream);
   else
-    launch_rmsnorm_out<bf16_t, bf16_t>(out, out_dtype, (bf16_t*)x, nullptr, w, row_idx, rows, dim, eps,
-                                       0, stream);
+    launch_rmsnorm_out<bf16_t, bf16_t>(out, out_dtype, (bf16_t*)x, nullptr, 0, 0, w, row_idx, rows, dim,
+                                       eps, 0, stream);
   PYLON_LAUNCHED("rmsnorm");
 }
 
 // resid (float) += delta, then out = rmsnorm(resid). With row_idx the sum is formed only
-// for the picked rows and resid is left untouched.
+// for the picked rows and resid is left untouched. delta may come as n_delta partial sums,
+// delta_stride elements apart, which are added up first.
 extern "C" int pylon_add_rmsnorm(void* out, int out_dtype, float* resid, const void* delta,
-                                 int delta_dtype, const float* w, const int* row_idx, int rows,
-                                 int dim, float eps, hipStream_t stream) {
+                                 int delta_dtype, int n_delta, long long delta_stride, const float* w,
+                                 const int* row_idx, int rows, int dim, float eps, hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(out_dtype), "add_rmsnorm: unknown out dtype");
   PYLON_REQUIRE(delta == nullptr || pylon_valid_dtype(delta_dtype), "add_rmsnorm: unknown delta dtype");
   PYLON_REQUIRE(rows >= 0 && dim > 0, "add_rmsnorm: bad sizes rows=%d dim=%d", rows, dim);
+  PYLON_REQUIRE(delta == nullptr || (n_delta >= 1 && n_delta <= 64), "add_rmsnorm: 1..64 partial sums");
   if (rows == 0) return 0;
   const int write_resid = (delta != nullptr && row_idx == nullptr) ? 1 : 0;
   if (delta == nullptr || delta_dtype == PYLON_F32)
-    launch_rmsnorm_out<float, float>(out, out_dtype, resid, (const float*)delta, w, row_idx, rows, dim,
-                                     eps, write_resid, stream);
+    launch_rmsnorm_out<float, float>(out, out_dtype, resid, (const float*)delta, n_delta, delta_stride,
+                                     w, row_idx, rows, dim, eps, write_resid, stream);
   else
-    launch_rmsnorm_out<float, bf16_t>(out, out_dtype, resid, (const bf16_t*)delta, w, row_idx, rows,
-                                      dim, eps, write_resid, stream);
+    launch_rmsnorm_out<float, bf16_t>(out, out_dtype, resid, (const bf16_t*)delta, n_delta,
+                                      delta_stride, w, row_idx, rows, dim, eps, write_resid, stream);
   PYLON_LAUNCHED("add_rmsnorm");
 }
 

@@ -98,6 +98,7 @@ class StepContext:
     max_count: int = 0
     max_len: int = 0
     decode_only: bool = False
+    fixed_shapes: bool = False  # launches must not depend on lengths (graph capture)
 
     def cache(self, cache_id: int) -> CacheView:
         return self.views[cache_id]

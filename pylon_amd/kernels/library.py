@@ -27,12 +27,14 @@ P, I, F, L = c_void_p, c_int, c_float, c_longlong
 _SIGNATURES = {
     "pylon_embed": [P, P, I, P, I, I, I, F, P],
     "pylon_rmsnorm": [P, I, P, I, P, P, I, I, F, P],
-    "pylon_add_rmsnorm": [P, I, P, P, I, P, P, I, I, F, P],
+    "pylon_add_rmsnorm": [P, I, P, P, I, I, L, P, P, I, I, F, P],
     "pylon_residual_add": [P, P, I, L, P],
     "pylon_silu_gate": [P, P, I, I, I, P],
     "pylon_qkv_prepare": [P, P, P, P, I, L, P, P, F, P, I, P, P, I, I, I, I, I, P],
     "pylon_paged_attention": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, P],
+    "pylon_attention_decode": [P, P, P, P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, P],
     "pylon_gemm_tiled": [P, I, P, I, P, I, I, I, I, L, L, L, P],
+    "pylon_gemm_skinny": [P, I, P, P, I, I, I, L, L, L, I, L, I, P],
     "pylon_argmax": [P, P, I, I, L, P],
     "pylon_sample": [P, P, I, I, L, P, P, P, P],
 }

@@ -81,13 +81,21 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``resid += delta`` (float32, in place) and the RMSNorm of the sum.
 
-    With ``row_idx`` only those rows are normed and ``resid`` is left as it is.
+    ``delta`` has the residual's shape, or is a stack ``[parts, tokens, dim]`` of partial
+    sums that are added up first.  With ``row_idx`` only those rows are normed and
+    ``resid`` is left as it is.
     """
     if resid.dim() != 2:
         raise KernelError("add_rmsnorm takes a 2-D residual")
     dim = resid.shape[1]
-    if delta is not None and delta.shape != resid.shape:
-        raise KernelError("add_rmsnorm: delta and resid differ in shape")
+    n_delta, delta_stride = 1, 0
+    if delta is not None:
+        if delta.dim() == 3:
+            n_delta, delta_stride = delta.shape[0], delta.shape[1] * delta.shape[2]
+            if delta.shape[1:] != resid.shape:
+                raise KernelError("add_rmsnorm: partial sums and resid differ in shape")
+        elif delta.shape != resid.shape:
+            raise KernelError("add_rmsnorm: delta and resid differ in shape")
     if weight.shape != (dim,):
         raise KernelError(f"add_rmsnorm: weight has shape {tuple(weight.shape)}, expected ({dim},)")
     rows = resid.shape[0] if row_idx is None else row_idx.numel()
@@ -97,7 +105,7 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
         raise KernelError("add_rmsnorm: out has the wrong shape or dtype")
     _lib.call("pylon_add_rmsnorm", _dev(out, "out"), dtype_code(out.dtype),
               _dev(resid, "resid", torch.float32), _dev(delta, "delta"),
-              dtype_code(delta.dtype) if delta is not None else F32,
+              dtype_code(delta.dtype) if delta is not None else F32, n_delta, delta_stride,
               _dev(weight, "weight", torch.float32), _dev(row_idx, "row_idx", torch.int32),
               rows, dim, float(eps), _stream())
     return out
@@ -196,6 +204,57 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     return out
 
 
+DECODE_HEAD_DIMS = (64, 128, 256)
+DECODE_MAX_TOKENS = 64
+
+
+def decode_attention_ok(q: torch.Tensor, k_cache: torch.Tensor) -> bool:
+    """Whether the key-split decode kernel takes this geometry."""
+    tokens, n_heads, head_dim = q.shape
+    n_kv_heads = k_cache.shape[2]
+    return (q.dtype == torch.bfloat16 and head_dim in DECODE_HEAD_DIMS and tokens <= DECODE_MAX_TOKENS
+            and n_heads % n_kv_heads == 0 and n_heads // n_kv_heads <= 16)
+
+
+def decode_splits(tokens: int, n_kv_heads: int, max_len: Optional[int]) -> int:
+    """Key ranges per (token, key/value head) so that a small batch still fills the chip."""
+    splits = max(1, min(16, 1024 // max(1, tokens * n_kv_heads)))
+    if max_len is not None:
+        splits = min(splits, max(1, (max_len + 63) // 64))
+    return splits
+
+
+def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                     block_table: torch.Tensor, tok_row: torch.Tensor, positions: torch.Tensor, *,
+                     page_size: int, window: Optional[int], scale: float, n_splits: int) -> torch.Tensor:
+    """Paged attention of a few bfloat16 query tokens, cut along the keys into
+    ``n_splits`` ranges whose partial results are merged."""
+    if q.dim() != 3 or not decode_attention_ok(q, k_cache):
+        raise KernelError("attention_decode does not take this geometry")
+    tokens, n_heads, head_dim = q.shape
+    pages, psize, n_kv_heads, hd = k_cache.shape
+    if psize != page_size or hd != head_dim or k_cache.shape != v_cache.shape:
+        raise KernelError("attention_decode: cache geometry does not match page_size/head_dim")
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        raise KernelError("attention_decode: q and the caches differ in dtype")
+    if pages * page_size >= 2 ** 31:
+        raise KernelError("attention_decode: the cache holds more slots than an int32 can index")
+    if tok_row.numel() != tokens or positions.numel() != tokens or block_table.dim() != 2:
+        raise KernelError("attention_decode: one row id and one position per token, and a 2-D table")
+    out = torch.empty_like(q)
+    part_acc = part_ml = None
+    if n_splits > 1:
+        part_acc = torch.empty((tokens * n_heads * n_splits * head_dim,), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((tokens * n_heads * n_splits * 2,), dtype=torch.float32, device=q.device)
+    _lib.call("pylon_attention_decode", _dev(out, "out"), _dev(part_acc, "part_acc"), _dev(part_ml, "part_ml"),
+              _dev(q, "q"), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
+              _dev(block_table, "block_table", torch.int32), block_table.shape[1],
+              _dev(tok_row, "tok_row", torch.int32), _dev(positions, "positions", torch.int32),
+              tokens, n_heads, n_kv_heads, head_dim, page_size, int(window or 0), float(scale),
+              int(n_splits), _stream())
+    return out
+
+
 def gemm_tiled(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.dtype] = None,
                out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ weight.T`` with float accumulation on the vector units (no matrix cores)."""
@@ -219,20 +278,79 @@ def gemm_tiled(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[tor
     return out
 
 
+SKINNY_ROWS = 64  # most rows of x the weight-streaming kernel takes
+
+
+def skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_ROWS
+            and weight.shape[1] % 8 == 0 and weight.stride(0) % 8 == 0 and x.stride(0) % 8 == 0)
+
+
+def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype = torch.bfloat16,
+                parts: int = 1, gated: bool = False) -> torch.Tensor:
+    """``x @ weight.T`` for at most 64 rows of bfloat16 ``x``, streaming ``weight`` once.
+
+    ``parts > 1`` cuts K into that many ranges and returns float32 partial results
+    ``[parts, M, N]`` for the consumer to add.  ``gated``: ``x`` is ``[M, 2K]`` and the
+    operand is ``silu(x[:, :K]) * x[:, K:]``, formed on the fly.
+    """
+    if x.dim() != 2 or weight.dim() != 2:
+        raise KernelError("gemm_skinny takes 2-D operands")
+    m, width = x.shape
+    n, k = weight.shape
+    if width != (2 * k if gated else k):
+        raise KernelError(f"gemm_skinny: cannot multiply {tuple(x.shape)} by the transpose of {tuple(weight.shape)}")
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise KernelError("gemm_skinny takes bfloat16 operands")
+    if not (x.is_cuda and weight.is_cuda) or x.stride(1) != 1 or weight.stride(1) != 1:
+        raise KernelError("gemm_skinny: operands must be on the GPU with contiguous rows")
+    if parts > 1:
+        out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
+    else:
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _lib.call("pylon_gemm_skinny", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), weight.data_ptr(),
+              m, n, k, x.stride(0), weight.stride(0), n, parts, m * n, 1 if gated else 0, _stream())
+    return out
+
+
+def k_parts(n: int, k: int) -> int:
+    """How many ranges to cut K into so that a matrix with few rows still fills the chip."""
+    tiles = (n + 15) // 16
+    parts = 1
+    while tiles * parts < 512 and parts < 8 and k // (parts * 2) >= 512:
+        parts *= 2
+    return parts
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """``x @ weight.T``.
 
-    bfloat16 by bfloat16 goes to the library matrix product (as the reference's
-    ``nn.Linear`` does); every pairing that involves float32 operands runs on the
-    exact tiled kernel, which never uses a reduced-precision matrix mode.
+    bfloat16 by bfloat16: up to 64 rows go to the weight-streaming kernel, more rows to
+    the library matrix product (as the reference's ``nn.Linear`` does).  Every pairing
+    that involves float32 operands runs on the exact tiled kernel, which never uses a
+    reduced-precision matrix mode.
     """
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
         if not x.is_cuda:
             raise KernelError("linear: operands must live on the GPU; there is no CPU path")
+        if skinny_ok(x, weight):
+            return gemm_skinny(x, weight, out_dtype=out_dtype)
         y = torch.nn.functional.linear(x, weight)
         return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
     return gemm_tiled(x, weight, out_dtype=out_dtype)
+
+
+def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype,
+                        gated: bool = False) -> torch.Tensor:
+    """A product whose result is about to be added to the residual stream: for few
+    rows it may come back as float32 partial sums ``[parts, M, N]``, which the fused
+    residual norm adds.  ``gated``: apply the gated activation to ``x`` first."""
+    if skinny_ok(x, weight):
+        return gemm_skinny(x, weight, out_dtype=out_dtype, parts=k_parts(*weight.shape), gated=gated)
+    if gated:
+        x = silu_gate(x)
+    return linear(x, weight, out_dtype=out_dtype)
 
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:

@@ -59,11 +59,19 @@ class Attention(Part):
             inv_freq=rotary[0] if rotary else None, rot_dim=rotary[1] if rotary else 0,
             positions=ctx.positions, slot_map=cache.slot_map, store_kv=stores,
         )
-        context = ops.paged_attention(
-            q, cache.k, cache.v, cache.block_table, ctx.tok_row, ctx.positions,
-            page_size=cache.page_size, window=spec.window, scale=spec.scale,
-        )
-        return ops.linear(context.view(tokens, spec.q_size), self.params["out"], out_dtype=self.dtype)
+        if ctx.decode_only and ops.decode_attention_ok(q, cache.k):
+            splits = ops.decode_splits(tokens, spec.n_kv_heads, None if ctx.fixed_shapes else ctx.max_len)
+            context = ops.attention_decode(
+                q, cache.k, cache.v, cache.block_table, ctx.tok_row, ctx.positions,
+                page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits,
+            )
+        else:
+            context = ops.paged_attention(
+                q, cache.k, cache.v, cache.block_table, ctx.tok_row, ctx.positions,
+                page_size=cache.page_size, window=spec.window, scale=spec.scale,
+            )
+        return ops.linear_for_residual(context.view(tokens, spec.q_size), self.params["out"],
+                                       out_dtype=self.dtype)
 
 
 register_part("mixer", "attention", Attention, replace=True)

@@ -8,13 +8,15 @@ Interfaces
 ----------
 norm          ``forward(x) -> y`` and ``add_forward(resid, delta, row_idx=None) -> y``:
               ``resid`` is the float32 residual stream, ``delta`` the previous part's
-              output (or None); the sum is formed in float32, stored back into
+              output (or None), either ``[tokens, dim]`` or a stack ``[parts, tokens, dim]``
+              of float32 partial sums still to be added up; the sum is formed in float32, stored back into
               ``resid`` (unless ``row_idx`` picks rows), and its norm is returned in
               the activation dtype.
 position      ``rotary() -> (inv_freq, rotary_dim) | None`` for encodings applied by
               rotating q and k, and ``check(max_position)``.
 mixer         ``cache_requirement() -> KVRequirement | StateRequirement | None`` and
-              ``forward(h, ctx, cache, stores) -> [tokens, hidden]``: ``cache`` is the
+              ``forward(h, ctx, cache, stores) -> [tokens, hidden]`` (or partial sums
+              ``[parts, tokens, hidden]`` in float32, see norm): ``cache`` is the
               view of the run's cache (its own, or the one it borrows); ``stores``
               says whether this run writes it.
 feed_forward  ``forward(h, ctx) -> [tokens, hidden]``.

@@ -22,8 +22,7 @@ class GatedFeedForward(Part):
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         gate_up = ops.linear(h, self.params["gate_up"], out_dtype=self.dtype)
-        hidden = ops.silu_gate(gate_up)
-        return ops.linear(hidden, self.params["down"], out_dtype=self.dtype)
+        return ops.linear_for_residual(gate_up, self.params["down"], out_dtype=self.dtype, gated=True)
 
 
 register_part("feed_forward", "gated_mlp", GatedFeedForward, replace=True)

@@ -119,6 +119,37 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops):
         assert torch.equal(part, whole[lo:hi])
 
 
+@pytest.mark.parametrize("shape", [(1, 96, 80), (8, 301, 176), (16, 130, 1000), (17, 64, 64),
+                                   (64, 2560 + 8, 512 + 24), (33, 48, 4096)])
+def test_gemm_skinny(ops, shape):
+    m, n, k = shape
+    a, w = rnd((m, k), 30, torch.bfloat16), rnd((n, k), 31, torch.bfloat16, 0.1)
+    want = f64(a) @ f64(w).T
+    for out_dtype in (torch.bfloat16, torch.float32):
+        got = ops.gemm_skinny(a.to(DEV), w.to(DEV), out_dtype=out_dtype)
+        assert got.shape == (m, n) and got.dtype == out_dtype
+        assert np.abs(f64(got) - want).max() <= tol(out_dtype, np.abs(want).max())
+    for parts in (2, 4, 7):
+        got = ops.gemm_skinny(a.to(DEV), w.to(DEV), parts=parts)
+        assert got.shape == (parts, m, n) and got.dtype == torch.float32
+        assert np.abs(f64(got).sum(0) - want).max() <= tol(torch.float32, np.abs(want).max())
+    # the same rows give the same bits whatever other rows share the launch
+    full = ops.gemm_skinny(a.to(DEV), w.to(DEV), out_dtype=torch.float32)
+    alone = ops.gemm_skinny(a[:1].contiguous().to(DEV), w.to(DEV), out_dtype=torch.float32)
+    assert torch.equal(alone, full[:1])
+    # gated input: silu(g) * u formed on the fly equals the separate activation kernel
+    gu = rnd((m, 2 * k), 32, torch.bfloat16, 2.0)
+    act = ops.silu_gate(gu.to(DEV))
+    sep = ops.gemm_skinny(act, w.to(DEV), out_dtype=torch.float32)
+    fused = ops.gemm_skinny(gu.to(DEV), w.to(DEV), out_dtype=torch.float32, gated=True)
+    assert torch.equal(sep, fused)
+    # through the dispatcher, and refused beyond 64 rows
+    assert torch.equal(ops.linear(a.to(DEV), w.to(DEV), out_dtype=torch.float32), full)
+    from pylon_amd.kernels import KernelError
+    with pytest.raises(KernelError, match="at most 64 rows"):
+        ops.gemm_skinny(torch.zeros((65, 64), dtype=torch.bfloat16, device=DEV), w[:, :64].contiguous().to(DEV))
+
+
 def plain_rope(x, pos, inv_freq, rot):
     # x: [..., d]; rotate the first `rot` elements, pairing i with i + rot/2
     ang = (np.float32(pos) * inv_freq.astype(np.float32)).astype(np.float64)
@@ -226,6 +257,55 @@ def test_paged_attention(ops, dtype, geom):
         vals = np.stack([vf[a, b] for a, b in idx], axis=1)
         want = plain_attention(f64(q)[i], keys, vals, scale, window)
         assert np.abs(f64(got)[i] - want).max() <= tol(dtype, max(1.0, np.abs(want).max())), (i, r, p)
+
+
+@pytest.mark.parametrize("geom", [(8, 2, 128, 64, None), (4, 4, 64, 16, None), (16, 1, 256, 32, 100),
+                                  (6, 2, 128, 256, None), (1, 1, 64, 16, 7)])
+@pytest.mark.parametrize("n_splits", [1, 3, 16])
+def test_attention_decode(ops, geom, n_splits):
+    nh, nkv, hd, page, window = geom
+    dtype = torch.bfloat16
+    lengths = [1, 15, 16, 17, 65, 300, 2 * page + 1, 700]
+    n_pages = sum(-(-n // page) for n in lengths) + 2
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(40)).tolist()
+    width = max(-(-n // page) for n in lengths)
+    table = torch.zeros((len(lengths), width), dtype=torch.int32)
+    cursor = 0
+    for r, n in enumerate(lengths):
+        for i in range(-(-n // page)):
+            table[r, i] = perm[cursor]
+            cursor += 1
+    kc = rnd((n_pages, page, nkv, hd), 41, dtype)
+    vc = rnd((n_pages, page, nkv, hd), 42, dtype)
+    # poison what no request holds and the slots past each request's end
+    held = set()
+    for r, n in enumerate(lengths):
+        for j in range(n):
+            held.add((int(table[r, j // page]), j % page))
+    for pg in range(n_pages):
+        for off in range(page):
+            if (pg, off) not in held:
+                kc[pg, off] = float("nan")
+                vc[pg, off] = float("nan")
+    rows = list(range(len(lengths)))[::-1]  # tokens in another order than the rows
+    positions = [lengths[r] - 1 for r in rows]
+    q = rnd((len(rows), nh, hd), 43, dtype)
+    scale = 1 / math.sqrt(hd)
+    args = (q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV),
+            torch.tensor(rows, dtype=torch.int32, device=DEV),
+            torch.tensor(positions, dtype=torch.int32, device=DEV))
+    got = ops.attention_decode(*args, page_size=page, window=window, scale=scale, n_splits=n_splits)
+    kf, vf = f64(kc), f64(vc)
+    for i, (r, p) in enumerate(zip(rows, positions)):
+        idx = [(int(table[r, j // page]), j % page) for j in range(p + 1)]
+        keys = np.stack([kf[a, b] for a, b in idx], axis=1)
+        vals = np.stack([vf[a, b] for a, b in idx], axis=1)
+        want = plain_attention(f64(q)[i], keys, vals, scale, window)
+        err = np.abs(f64(got)[i] - want).max()
+        assert err <= tol(dtype, max(1.0, np.abs(want).max())), (i, r, p, err)
+    # the general kernel agrees to rounding
+    ref = ops.paged_attention(*args, page_size=page, window=window, scale=scale)
+    assert float((got.float() - ref.float()).abs().max()) <= 2e-2
 
 
 def test_attention_finds_one_far_key_among_hundreds(ops):
