@@ -56,8 +56,8 @@ def build_runner(layers: int, dtype: str, max_requests: int, num_pages: int, gra
     model = Model(arch.model_spec(cfg), dtype=resolve_dtype(dtype), device="cuda:0")
     model.init_random(seed=0)
     runner = Runner(model, page_size=PAGE_SIZE, num_pages=num_pages, max_requests=max_requests)
-    if graphs and hasattr(runner, "enable_graphs"):
-        runner.enable_graphs()
+    if graphs:
+        runner.enable_graphs(max_requests, max_tokens_per_request=CONTEXT_LENGTH)
     torch.cuda.synchronize()
     return runner, cfg
 
@@ -189,7 +189,7 @@ def main() -> int:
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
             "global_batch": args.batch, "seq_len": PROMPT_LEN, "new_tokens": steps,
             "context_length": CONTEXT_LENGTH, "page_size": PAGE_SIZE, "prefill_tokens": PREFILL_TOKENS,
-            "hip_graphs": bool(getattr(runner, "graphs", None)), "parallelism": "single-gpu",
+            "hip_graphs": runner.graphs is not None, "parallelism": "single-gpu",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_BYTES_PER_S / 1e9,
                      "unit": "GB/s", "frac": round(achieved / HBM_BYTES_PER_S, 4)},

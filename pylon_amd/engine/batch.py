@@ -130,7 +130,7 @@ def plan_layout(tokens: int, rows: int, n_logits: int, n_groups: int, width: int
 
 def build_step(entries: Seq[StepEntry], manager: CacheManager, arena: MetadataArena, *,
                vocab_size: int, width: Optional[int] = None,
-               device_block: Optional[torch.Tensor] = None) -> StepContext:
+               device_block: Optional[torch.Tensor] = None, fixed_shapes: bool = False) -> StepContext:
     """Check the entries, take the pages they need, and put the step's metadata on the
     device.  Raises before touching the cache if any entry is malformed; raises
     :class:`~pylon_amd.cache.pages.OutOfPages` (cache untouched) if pages run short."""
@@ -209,4 +209,5 @@ def build_step(entries: Seq[StepEntry], manager: CacheManager, arena: MetadataAr
         logit_idx=dev("logit_idx") if logit_list else None, n_logits=len(logit_list),
         views=views, counts=counts, starts=starts, max_count=int(counts.max()),
         max_len=int(seq_lens.max()), decode_only=bool((counts == 1).all()),
+        fixed_shapes=fixed_shapes,
     )

@@ -1,0 +1,86 @@
+"""HIP graph replay of decode-only steps.
+
+As in the reference (/root/reference/src/pylon/decode/graph.py:71-242) there is one graph
+per batch size, captured over static buffers; a replay fills the buffers and launches the
+graph; a batch size without a graph, or whose capture failed, runs kernel by kernel, and a
+failed capture is not tried again.  Differences: the static buffers are one packed block
+of metadata (filled by the same code that prepares any other step), graphs are captured
+the first time a batch size is seen rather than all at start-up, and a batch is never
+padded to a larger captured size.
+
+The launches recorded in a graph must not depend on the requests' lengths: the block
+table has a fixed width, and the decode attention kernel cuts keys into a number of
+ranges that depends on the batch size only.
+"""
+from __future__ import annotations
+
+import logging
+from typing import Dict, Optional, Sequence as Seq, Tuple
+
+import torch
+
+from .batch import StepEntry, build_step, plan_layout
+
+logger = logging.getLogger("pylon")
+
+
+class DecodeGraphs:
+    def __init__(self, runner, *, max_batch: int, max_pages_per_request: int) -> None:
+        self.runner = runner
+        self.max_batch = max_batch
+        self.width = max_pages_per_request
+        self.pool = torch.cuda.graph_pool_handle()
+        self.captured: Dict[int, Tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor]] = {}
+        self.failed = set()
+        self.replays = 0
+
+    def captured_sizes(self):
+        return tuple(sorted(self.captured))
+
+    def wants(self, entries: Seq[StepEntry]) -> bool:
+        """A decode-only step: one token per request, each wanting its logits."""
+        rows = len(entries)
+        if rows > self.max_batch or rows in self.failed:
+            return False
+        page = self.runner.manager.page_size
+        for e in entries:
+            if len(e.tokens) != 1 or list(e.want) != [0]:
+                return False
+            if e.seq.length + 1 > self.width * page:
+                return False  # longer than the captured block table: run kernel by kernel
+        return True
+
+    def run(self, entries: Seq[StepEntry]) -> Optional[torch.Tensor]:
+        """Replay (capturing first if need be).  Returns None if this batch size has no
+        graph; the caller then runs the step kernel by kernel.  The cache is reserved and
+        committed here exactly as an ordinary step does."""
+        runner = self.runner
+        rows = len(entries)
+        manager = runner.manager
+        pairs = [(e.seq, 1) for e in entries]
+        entry = self.captured.get(rows)
+        if entry is None:
+            _, size = plan_layout(rows, rows, rows, len(manager.groups), self.width)
+            block = torch.empty(size, dtype=torch.int32, device=runner.model.device)
+            ctx = build_step(entries, manager, runner.arena, vocab_size=runner.model.spec.vocab_size,
+                             width=self.width, device_block=block, fixed_shapes=True)
+            try:
+                torch.cuda.synchronize(runner.model.device)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, pool=self.pool):
+                    logits = runner.model.step(ctx)
+            except Exception:  # noqa: BLE001 - a failed capture leaves this size to eager steps
+                logger.exception("decode_graph_capture_failed batch_size=%s", rows)
+                self.failed.add(rows)
+                manager.cancel(pairs)
+                return None
+            self.captured[rows] = (graph, block, logits)
+            graph.replay()  # capture records only; this runs the step
+        else:
+            graph, block, logits = entry
+            build_step(entries, manager, runner.arena, vocab_size=runner.model.spec.vocab_size,
+                       width=self.width, device_block=block, fixed_shapes=True)
+            graph.replay()
+        self.replays += 1
+        manager.commit(pairs)
+        return logits

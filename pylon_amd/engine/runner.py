@@ -85,7 +85,21 @@ class Runner:
         runner = cls(model, page_size=config.page_size, num_pages=int(num_pages),
                      max_requests=config.max_batch_size)
         runner.config = model_config
+        if config.cuda_graphs:
+            runner.enable_graphs(config.max_batch_size)
         return runner
+
+    def enable_graphs(self, max_batch: Optional[int] = None, max_tokens_per_request: Optional[int] = None) -> None:
+        """Replay decode-only steps of up to ``max_batch`` requests from HIP graphs.
+        ``max_tokens_per_request`` bounds the lengths a graph serves (longer requests run
+        kernel by kernel); by default whatever the page pool could hold."""
+        from .graphs import DecodeGraphs
+
+        page = self.manager.page_size
+        limit = max_tokens_per_request or self.model.spec.max_positions or self.manager.capacity_tokens
+        limit = min(limit, self.manager.capacity_tokens)
+        self.graphs = DecodeGraphs(self, max_batch=max_batch or self.manager.slots.max_slots,
+                                   max_pages_per_request=-(-limit // page))
 
     def synchronize(self) -> None:
         torch.cuda.synchronize(self.model.device)
@@ -114,6 +128,10 @@ class Runner:
                     raise ValueError(
                         f"The model supports at most {max_positions:,} tokens per request."
                     )
+        if self.graphs is not None and self.graphs.wants(entries):
+            logits = self.graphs.run(entries)
+            if logits is not None:
+                return logits
         ctx = build_step(entries, self.manager, self.arena, vocab_size=self.model.spec.vocab_size)
         pairs = [(e.seq, len(e.tokens)) for e in entries]
         try:

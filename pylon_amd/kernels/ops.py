@@ -287,19 +287,21 @@ def skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
 
 
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype = torch.bfloat16,
-                parts: int = 1, gated: bool = False) -> torch.Tensor:
+                parts: int = 1, glu: bool = False) -> torch.Tensor:
     """``x @ weight.T`` for at most 64 rows of bfloat16 ``x``, streaming ``weight`` once.
 
     ``parts > 1`` cuts K into that many ranges and returns float32 partial results
-    ``[parts, M, N]`` for the consumer to add.  ``gated``: ``x`` is ``[M, 2K]`` and the
-    operand is ``silu(x[:, :K]) * x[:, K:]``, formed on the fly.
+    ``[parts, M, N]`` for the consumer to add.  ``glu``: ``weight`` is a fused
+    ``[2N, K]`` gate/up matrix and the result is ``silu(x @ gate.T) * (x @ up.T)``.
     """
-    if x.dim() != 2 or weight.dim() != 2:
-        raise KernelError("gemm_skinny takes 2-D operands")
-    m, width = x.shape
-    n, k = weight.shape
-    if width != (2 * k if gated else k):
+    if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
         raise KernelError(f"gemm_skinny: cannot multiply {tuple(x.shape)} by the transpose of {tuple(weight.shape)}")
+    m, k = x.shape
+    n = weight.shape[0]
+    if glu:
+        if n % 2:
+            raise KernelError("gemm_skinny: a fused gate/up matrix has an even number of rows")
+        n //= 2
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
         raise KernelError("gemm_skinny takes bfloat16 operands")
     if not (x.is_cuda and weight.is_cuda) or x.stride(1) != 1 or weight.stride(1) != 1:
@@ -309,7 +311,7 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype
     else:
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     _lib.call("pylon_gemm_skinny", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), weight.data_ptr(),
-              m, n, k, x.stride(0), weight.stride(0), n, parts, m * n, 1 if gated else 0, _stream())
+              m, n, k, x.stride(0), weight.stride(0), n, parts, m * n, 1 if glu else 0, _stream())
     return out
 
 
@@ -341,16 +343,20 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.d
     return gemm_tiled(x, weight, out_dtype=out_dtype)
 
 
-def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype,
-                        gated: bool = False) -> torch.Tensor:
+def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:
     """A product whose result is about to be added to the residual stream: for few
     rows it may come back as float32 partial sums ``[parts, M, N]``, which the fused
-    residual norm adds.  ``gated``: apply the gated activation to ``x`` first."""
+    residual norm adds."""
     if skinny_ok(x, weight):
-        return gemm_skinny(x, weight, out_dtype=out_dtype, parts=k_parts(*weight.shape), gated=gated)
-    if gated:
-        x = silu_gate(x)
+        return gemm_skinny(x, weight, out_dtype=out_dtype, parts=k_parts(*weight.shape))
     return linear(x, weight, out_dtype=out_dtype)
+
+
+def linear_glu(x: torch.Tensor, gate_up: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:
+    """``silu(x @ gate.T) * (x @ up.T)`` for a fused ``[2I, K]`` gate/up matrix."""
+    if skinny_ok(x, gate_up):
+        return gemm_skinny(x, gate_up, out_dtype=out_dtype, glu=True)
+    return silu_gate(linear(x, gate_up, out_dtype=out_dtype))
 
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:

@@ -21,8 +21,8 @@ class GatedFeedForward(Part):
         self.add_param("down", (spec.hidden_size, spec.intermediate_size), dtype, device)
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
-        gate_up = ops.linear(h, self.params["gate_up"], out_dtype=self.dtype)
-        return ops.linear_for_residual(gate_up, self.params["down"], out_dtype=self.dtype, gated=True)
+        hidden = ops.linear_glu(h, self.params["gate_up"], out_dtype=self.dtype)
+        return ops.linear_for_residual(hidden, self.params["down"], out_dtype=self.dtype)
 
 
 register_part("feed_forward", "gated_mlp", GatedFeedForward, replace=True)

@@ -1,0 +1,86 @@
+"""Decode-only steps replayed from HIP graphs give what the same steps give kernel by
+kernel, over many replays with other work and synchronisations in between, while requests
+join and leave (so batch sizes change) and pages are used again."""
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import CONFIGS, make_model_folder, random_tokens, read_folder
+from tests.plain import qwen3 as plain
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype,name", [("float32", "A"), ("bfloat16", "B"), ("bfloat16", "C")])
+def test_graph_replay_equals_eager_steps(tmp_path, dtype, name):
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from pylon_amd.engine import Runner, StepEntry
+
+    folder = make_model_folder(tmp_path, name, dtype=dtype, std=0.08)
+    cfg, weights = read_folder(folder)
+    vocab = cfg["vocab_size"]
+    prompts = {f"g{i}": random_tokens(vocab, n, 300 + i) for i, n in enumerate((3, 20, 33, 9))}
+    decode = {rid: random_tokens(vocab, 40, 400 + i) for i, rid in enumerate(prompts)}
+
+    def run(graphs):
+        runner = Runner.from_folder(folder, dtype=dtype, page_size=16, num_pages=24, max_requests=4)
+        if graphs:
+            runner.enable_graphs(4, max_tokens_per_request=96)
+        live, rows = {}, {rid: [] for rid in prompts}
+        order = list(prompts)
+        for step in range(40):
+            # requests join one after the other and leave at different times
+            if step % 3 == 0 and order:
+                rid = order.pop(0)
+                live[rid] = runner.open(rid)
+                out = runner.step([StepEntry(live[rid], prompts[rid], [len(prompts[rid]) - 1])])
+                rows[rid].append(out[0].cpu().numpy())
+            torch.cuda.synchronize()
+            entries, who = [], []
+            for rid, seq in live.items():
+                i = seq.length - len(prompts[rid])
+                entries.append(StepEntry(seq, [decode[rid][i]], [0]))
+                who.append(rid)
+            if entries:
+                out = runner.step(entries).cpu().numpy()
+                for r, rid in enumerate(who):
+                    rows[rid].append(out[r])
+            for rid in list(live):
+                done = live[rid].length - len(prompts[rid])
+                if done >= (12, 40, 25, 31)[list(prompts).index(rid)]:
+                    runner.close(live.pop(rid))
+            runner.manager.check()
+        return runner, {rid: np.stack(r) for rid, r in rows.items()}
+
+    eager_runner, eager = run(False)
+    graph_runner, graphed = run(True)
+    assert graph_runner.graphs.replays > 30 and set(graph_runner.graphs.captured_sizes()) >= {1, 2, 3}
+    bound = 0.0 if dtype == "float32" else 1e-2
+    for rid in prompts:
+        assert eager[rid].shape == graphed[rid].shape
+        scale = np.abs(eager[rid]).max()
+        assert np.abs(eager[rid] - graphed[rid]).max() <= bound * scale, rid
+        # and both are the plain model's logits
+        n = eager[rid].shape[0]
+        toks = prompts[rid] + decode[rid][: n - 1]
+        want = plain.forward(weights, cfg, toks)[len(prompts[rid]) - 1:]
+        tol = 2e-5 if dtype == "float32" else 2e-2
+        assert np.abs(graphed[rid] - want).max() <= tol * np.abs(want).max(), rid
+
+
+def test_a_request_longer_than_the_captured_table_runs_eagerly(tmp_path):
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from pylon_amd.engine import Runner, StepEntry
+
+    folder = make_model_folder(tmp_path, "C", dtype="bfloat16", std=0.08)
+    cfg, _ = read_folder(folder)
+    runner = Runner.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=12, max_requests=2)
+    runner.enable_graphs(2, max_tokens_per_request=32)
+    seq = runner.open("x")
+    toks = random_tokens(cfg["vocab_size"], 60, 1)
+    runner.step([StepEntry(seq, toks[:28], [])])
+    for t in toks[28:40]:
+        runner.step([StepEntry(seq, [t], [0])])
+    assert runner.graphs.replays == 4 and seq.length == 40  # positions 28..31 fit the table

@@ -120,7 +120,7 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops):
 
 
 @pytest.mark.parametrize("shape", [(1, 96, 80), (8, 301, 176), (16, 130, 1000), (17, 64, 64),
-                                   (64, 2560 + 8, 512 + 24), (33, 48, 4096)])
+                                   (64, 2560 + 8, 512 + 24), (33, 48, 4096), (8, 72, 9728)])
 def test_gemm_skinny(ops, shape):
     m, n, k = shape
     a, w = rnd((m, k), 30, torch.bfloat16), rnd((n, k), 31, torch.bfloat16, 0.1)
@@ -137,12 +137,15 @@ def test_gemm_skinny(ops, shape):
     full = ops.gemm_skinny(a.to(DEV), w.to(DEV), out_dtype=torch.float32)
     alone = ops.gemm_skinny(a[:1].contiguous().to(DEV), w.to(DEV), out_dtype=torch.float32)
     assert torch.equal(alone, full[:1])
-    # gated input: silu(g) * u formed on the fly equals the separate activation kernel
-    gu = rnd((m, 2 * k), 32, torch.bfloat16, 2.0)
-    act = ops.silu_gate(gu.to(DEV))
-    sep = ops.gemm_skinny(act, w.to(DEV), out_dtype=torch.float32)
-    fused = ops.gemm_skinny(gu.to(DEV), w.to(DEV), out_dtype=torch.float32, gated=True)
-    assert torch.equal(sep, fused)
+    # gated epilogue over a fused gate/up matrix equals product, then the activation kernel
+    if n % 2 == 0:
+        both = ops.gemm_skinny(a.to(DEV), w.to(DEV), out_dtype=torch.float32)
+        g, u = f64(both)[:, : n // 2], f64(both)[:, n // 2:]
+        want_glu = g / (1 + np.exp(-g)) * u
+        fused = ops.gemm_skinny(a.to(DEV), w.to(DEV), glu=True)
+        assert fused.shape == (m, n // 2)
+        assert np.abs(f64(fused) - want_glu).max() <= tol(torch.bfloat16, np.abs(want_glu).max())
+        assert torch.equal(ops.linear_glu(a.to(DEV), w.to(DEV), out_dtype=torch.bfloat16), fused)
     # through the dispatcher, and refused beyond 64 rows
     assert torch.equal(ops.linear(a.to(DEV), w.to(DEV), out_dtype=torch.float32), full)
     from pylon_amd.kernels import KernelError
