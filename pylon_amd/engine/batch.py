@@ -99,9 +99,32 @@ class StepContext:
     max_len: int = 0
     decode_only: bool = False
     fixed_shapes: bool = False  # launches must not depend on lengths (graph capture)
+    _tiles: Dict[int, torch.Tensor] = field(default_factory=dict)
 
     def cache(self, cache_id: int) -> CacheView:
         return self.views[cache_id]
+
+    def token_tiles(self, tokens_per_tile: int) -> torch.Tensor:
+        """int32 ``[n, 4]`` on the device: the step's tokens cut into runs of at most
+        ``tokens_per_tile`` consecutive tokens of one row, as (index of the first token,
+        count, row, position of the first token), longest context first so that the
+        heaviest tiles start first."""
+        tiles = self._tiles.get(tokens_per_tile)
+        if tiles is None:
+            per_row = -(-self.counts // tokens_per_tile)
+            row = np.repeat(np.arange(self.rows, dtype=np.int64), per_row)
+            first_of_row = np.zeros(self.rows + 1, dtype=np.int64)
+            np.cumsum(per_row, out=first_of_row[1:])
+            within = (np.arange(int(per_row.sum()), dtype=np.int64) - first_of_row[row]) * tokens_per_tile
+            count = np.minimum(tokens_per_tile, self.counts[row] - within)
+            starts = np.zeros(self.rows + 1, dtype=np.int64)
+            np.cumsum(self.counts, out=starts[1:])
+            table = np.stack([starts[row] + within, count, row, self.starts[row] + within], axis=1)
+            order = np.argsort(-(table[:, 3] + table[:, 1]), kind="stable")
+            host = torch.from_numpy(np.ascontiguousarray(table[order].astype(np.int32)))
+            tiles = host.to(self.token_ids.device)
+            self._tiles[tokens_per_tile] = tiles
+        return tiles
 
 
 def plan_layout(tokens: int, rows: int, n_logits: int, n_groups: int, width: int) -> Tuple[Dict[str, Tuple[int, int]], int]:

@@ -255,6 +255,42 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     return out
 
 
+PREFILL_ROWS = 128  # (token, head) query rows one workgroup of the prefill kernel takes
+
+
+def prefill_attention_ok(q: torch.Tensor, k_cache: torch.Tensor) -> bool:
+    tokens, n_heads, head_dim = q.shape
+    n_kv_heads = k_cache.shape[2]
+    return (q.dtype == torch.bfloat16 and head_dim in DECODE_HEAD_DIMS and n_heads % n_kv_heads == 0
+            and n_heads // n_kv_heads <= PREFILL_ROWS)
+
+
+def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      block_table: torch.Tensor, tiles: torch.Tensor, *, page_size: int,
+                      window: Optional[int], scale: float) -> torch.Tensor:
+    """Paged causal attention of bfloat16 prompt portions on the matrix cores.  ``tiles`` is
+    int32 ``[n, 4]``: first token index, token count, block-table row and first position of
+    runs of at most ``128 // group`` consecutive tokens of one request."""
+    if q.dim() != 3 or not prefill_attention_ok(q, k_cache):
+        raise KernelError("attention_prefill does not take this geometry")
+    tokens, n_heads, head_dim = q.shape
+    pages, psize, n_kv_heads, hd = k_cache.shape
+    if psize != page_size or hd != head_dim or k_cache.shape != v_cache.shape:
+        raise KernelError("attention_prefill: cache geometry does not match page_size/head_dim")
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        raise KernelError("attention_prefill: q and the caches differ in dtype")
+    if pages * page_size >= 2 ** 31:
+        raise KernelError("attention_prefill: the cache holds more slots than an int32 can index")
+    if tiles.dim() != 2 or tiles.shape[1] != 4 or block_table.dim() != 2:
+        raise KernelError("attention_prefill: tiles must be [n, 4] and the block table 2-D")
+    out = torch.empty_like(q)
+    _lib.call("pylon_attention_prefill", _dev(out, "out"), _dev(q, "q"), _dev(k_cache, "k_cache"),
+              _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
+              _dev(tiles, "tiles", torch.int32), tiles.shape[0], n_heads, n_kv_heads, head_dim, page_size,
+              int(window or 0), float(scale), _stream())
+    return out
+
+
 def gemm_tiled(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.dtype] = None,
                out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ weight.T`` with float accumulation on the vector units (no matrix cores)."""

@@ -65,6 +65,12 @@ class Attention(Part):
                 q, cache.k, cache.v, cache.block_table, ctx.tok_row, ctx.positions,
                 page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits,
             )
+        elif ops.prefill_attention_ok(q, cache.k):
+            tiles = ctx.token_tiles(ops.PREFILL_ROWS // (spec.n_heads // spec.n_kv_heads))
+            context = ops.attention_prefill(
+                q, cache.k, cache.v, cache.block_table, tiles,
+                page_size=cache.page_size, window=spec.window, scale=spec.scale,
+            )
         else:
             context = ops.paged_attention(
                 q, cache.k, cache.v, cache.block_table, ctx.tok_row, ctx.positions,

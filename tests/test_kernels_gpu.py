@@ -311,6 +311,66 @@ def test_attention_decode(ops, geom, n_splits):
     assert float((got.float() - ref.float()).abs().max()) <= 2e-2
 
 
+@pytest.mark.parametrize("geom", [(8, 2, 128, 64, None), (4, 4, 64, 16, None), (12, 2, 128, 32, 100),
+                                  (5, 1, 256, 16, None), (3, 3, 64, 256, 37), (16, 1, 128, 64, None)])
+def test_attention_prefill(ops, geom):
+    """Portions of several requests at once: starting inside a page, a one-token portion, a
+    portion with earlier context; pages in scrambled order, everything unheld poisoned."""
+    nh, nkv, hd, page, window = geom
+    dtype = torch.bfloat16
+    group = nh // nkv
+    # (tokens cached before, tokens of this portion)
+    portions = [(0, 70), (33, 1), (100, 45), (0, 3), (2 * page - 1, 130), (5, 64)]
+    lengths = [a + b for a, b in portions]
+    n_pages = sum(-(-n // page) for n in lengths) + 2
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(50)).tolist()
+    width = max(-(-n // page) for n in lengths)
+    table = torch.zeros((len(lengths), width), dtype=torch.int32)
+    cursor = 0
+    for r, n in enumerate(lengths):
+        for i in range(-(-n // page)):
+            table[r, i] = perm[cursor]
+            cursor += 1
+    kc = rnd((n_pages, page, nkv, hd), 51, dtype)
+    vc = rnd((n_pages, page, nkv, hd), 52, dtype)
+    held = {(int(table[r, j // page]), j % page) for r, n in enumerate(lengths) for j in range(n)}
+    for pg in range(n_pages):
+        for off in range(page):
+            if (pg, off) not in held:
+                kc[pg, off] = float("nan")
+                vc[pg, off] = float("nan")
+    tok_row, positions, tiles = [], [], []
+    per_tile = ops.PREFILL_ROWS // group
+    for r, (before, count) in enumerate(portions):
+        for lo in range(0, count, per_tile):
+            tiles.append((len(tok_row) + lo, min(per_tile, count - lo), r, before + lo))
+        tok_row += [r] * count
+        positions += list(range(before, before + count))
+    tiles = tiles[::-1]  # any order
+    q = rnd((len(tok_row), nh, hd), 53, dtype)
+    scale = 1 / math.sqrt(hd)
+    got = ops.attention_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV),
+                                torch.tensor(tiles, dtype=torch.int32, device=DEV),
+                                page_size=page, window=window, scale=scale)
+    assert not torch.isnan(got.float()).any()
+    kf, vf = f64(kc), f64(vc)
+    worst = 0.0
+    for i, (r, p) in enumerate(zip(tok_row, positions)):
+        idx = [(int(table[r, j // page]), j % page) for j in range(p + 1)]
+        keys = np.stack([kf[a, b] for a, b in idx], axis=1)
+        vals = np.stack([vf[a, b] for a, b in idx], axis=1)
+        want = plain_attention(f64(q)[i], keys, vals, scale, window)
+        err = np.abs(f64(got)[i] - want).max()
+        # probabilities are rounded to bfloat16 before they weigh the values
+        assert err <= 2 * tol(dtype, max(1.0, np.abs(want).max())), (i, r, p, err)
+        worst = max(worst, err)
+    ref = ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV),
+                              torch.tensor(tok_row, dtype=torch.int32, device=DEV),
+                              torch.tensor(positions, dtype=torch.int32, device=DEV),
+                              page_size=page, window=window, scale=scale)
+    assert float((got.float() - ref.float()).abs().max()) <= 3e-2
+
+
 def test_attention_finds_one_far_key_among_hundreds(ops):
     # Random keys would hide a key that is skipped; here one far key matches the query
     # exactly and strongly, so the output must be (almost) that key's value.
