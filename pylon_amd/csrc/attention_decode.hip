@@ -1,72 +1,79 @@
 // Paged attention for steps with few query tokens (decode): bfloat16, head sizes 64, 128
 // and 256, any grouping of up to 16 query heads per key/value head.
-// It is bound by reading each request's keys and values once, so the work is cut along
-// the keys: one wavefront takes one (token, key/value head, range of keys), handles all
-// query heads of the group together, and leaves a partial result (running maximum, sum
-// and weighted values in float); a second kernel merges the ranges of a token's head.
+//
+// A decode step waits on memory latency more than on bandwidth, so the kernel is built to
+// make few trips to memory.  One workgroup takes one (token, key/value head) and handles
+// all query heads of the group together.  Its wavefronts cut the token's keys into equal
+// ranges; a wave issues the loads of up to 64 keys and of their values all at once, then
+// computes.  The waves' partial results (running maximum, sum, weighted values, in float)
+// meet in LDS and are merged in the order of the ranges, so no partial result ever goes
+// through global memory and there is no second kernel.
 //
 // Scores come from the 16x16x32 bf16 matrix instruction with 16 keys as rows and the
 // group's query heads as columns (unused columns are zero).  The weighted sum of values
-// runs on the vector units with one lane per pair of output elements, so values are read
-// as whole contiguous rows.  Softmax statistics are float throughout.
+// runs on the vector units with each lane owning head_dim/64 consecutive output elements,
+// so values are read as whole contiguous rows.  Softmax statistics are float throughout.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 #define AD_MAX_GROUP 16
-#define AD_TILE 16  // keys per score tile
+#define AD_TILE 16   // keys per score tile
+#define AD_SUPER 64  // keys whose loads are in flight together (four score tiles)
+#define AD_MAX_WAVES 16
 
-// A lane owns EPL consecutive elements of a head (EPL = head_dim / 64).
+// EPL consecutive bfloat16 elements kept packed (two per register) until they are used.
 template <int EPL>
-__device__ __forceinline__ void load_bf16_elems(const uint16_t* p, float* v);
-template <>
-__device__ __forceinline__ void load_bf16_elems<1>(const uint16_t* p, float* v) {
-  v[0] = bf16_bits_to_float(*p);
-}
-template <>
-__device__ __forceinline__ void load_bf16_elems<2>(const uint16_t* p, float* v) {
-  const uint32_t two = *reinterpret_cast<const uint32_t*>(p);
-  v[0] = __uint_as_float(two << 16);
-  v[1] = __uint_as_float(two & 0xffff0000u);
-}
-template <>
-__device__ __forceinline__ void load_bf16_elems<4>(const uint16_t* p, float* v) {
-  const uint2 four = *reinterpret_cast<const uint2*>(p);
-  v[0] = __uint_as_float(four.x << 16);
-  v[1] = __uint_as_float(four.x & 0xffff0000u);
-  v[2] = __uint_as_float(four.y << 16);
-  v[3] = __uint_as_float(four.y & 0xffff0000u);
-}
-template <int EPL>
-__device__ __forceinline__ void store_bf16_elems(uint16_t* p, const float* v) {
-#pragma unroll
-  for (int i = 0; i < EPL; ++i) p[i] = float_to_bf16_bits(v[i]);
-}
+struct PackedElems {
+  uint32_t raw[(EPL + 1) / 2];
+  __device__ __forceinline__ void load(const uint16_t* p) {
+    if (EPL == 1) {
+      raw[0] = *p;
+    } else if (EPL == 2) {
+      raw[0] = *reinterpret_cast<const uint32_t*>(p);
+    } else {
+      const uint2 four = *reinterpret_cast<const uint2*>(p);
+      raw[0] = four.x;
+      raw[(EPL + 1) / 2 - 1] = four.y;
+    }
+  }
+  __device__ __forceinline__ float get(int i) const {
+    const uint32_t word = raw[i / 2];
+    return (i & 1) ? __uint_as_float(word & 0xffff0000u) : __uint_as_float(word << 16);
+  }
+};
 
-template <int EPL, int KSTEPS>  // EPL = head_dim / 64, KSTEPS = head_dim / 32
-__global__ __launch_bounds__(PYLON_WAVE) void attention_decode_kernel(
-    uint16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
-    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
+// EPL = head_dim / 64, KSTEPS = head_dim / 32, GP = heads per group rounded up to 1, 2, 4, 8, 16
+template <int EPL, int KSTEPS, int GP>
+__global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_kernel(
+    uint16_t* __restrict__ out, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tok_row, const int* __restrict__ positions, int n_heads, int n_kv_heads,
-    int page_size, int window, float scale, int n_splits) {
+    int page_size, int window, float scale) {
   constexpr int HD = EPL * 64;
-  __shared__ float p_tile[AD_TILE][AD_MAX_GROUP];
-  const int lane = threadIdx.x;
+  constexpr int TILES = AD_SUPER / AD_TILE;
+  // per wave: probabilities of the keys in flight; then the waves' partial results
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int n_waves = blockDim.x / PYLON_WAVE;
+  const int lane = threadIdx.x & (PYLON_WAVE - 1);
+  const int wave = threadIdx.x / PYLON_WAVE;
+  float(*p_tile)[GP] = reinterpret_cast<float(*)[GP]>(lds + wave * AD_SUPER * GP);
+  float* part_acc = lds + n_waves * AD_SUPER * GP;  // [wave][GP][HD]
+  float* part_ml = part_acc + n_waves * GP * HD;    // [wave][GP][2]
   const int col = lane & 15, grp = lane >> 4;
-  const int split = blockIdx.x, kvh = blockIdx.y, t = blockIdx.z;
+  const int kvh = blockIdx.x, t = blockIdx.y;
   const int group = n_heads / n_kv_heads;
   const int pos = positions[t];
   const int* table = block_table + static_cast<size_t>(tok_row[t]) * table_width;
 
-  // the keys of this split
+  // the keys of this wave
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int n_keys = pos + 1 - first;
-  int per_split = (n_keys + n_splits - 1) / n_splits;
-  per_split = (per_split + AD_TILE - 1) / AD_TILE * AD_TILE;
-  const int k_begin = first + split * per_split;
-  int k_end = k_begin + per_split;
+  int per_wave = (n_keys + n_waves - 1) / n_waves;
+  per_wave = (per_wave + AD_TILE - 1) / AD_TILE * AD_TILE;
+  const int k_begin = first + wave * per_wave;
+  int k_end = k_begin + per_wave;
   if (k_end > pos + 1) k_end = pos + 1;
 
   // query fragments: column `col` is head kvh*group + col of the token
@@ -86,162 +93,166 @@ __global__ __launch_bounds__(PYLON_WAVE) void attention_decode_kernel(
   }
 
   float m_run = -INFINITY, l_run = 0.f;  // for head `col` (same in the 4 lanes that share it)
-  float acc[AD_MAX_GROUP][EPL];  // only the first `group` rows are used
+  float acc[GP][EPL];                    // rows past `group` hold nothing of use
 #pragma unroll
-  for (int h = 0; h < AD_MAX_GROUP; ++h)
+  for (int h = 0; h < GP; ++h)
 #pragma unroll
     for (int i = 0; i < EPL; ++i) acc[h][i] = 0.f;
 
-  for (int base = k_begin; base < k_end; base += AD_TILE) {
-    // row `col` of the tile is key base + col; rows past the end repeat the last key
-    const int key = (base + col < k_end) ? base + col : k_end - 1;
-    const int phys = table[key / page_size] * page_size + key % page_size;
-    const uint16_t* krow = k_cache + (static_cast<size_t>(phys) * n_kv_heads + kvh) * HD;
-    floatx4 s = {0.f, 0.f, 0.f, 0.f};
+  for (int base = k_begin; base < k_end; base += AD_SUPER) {
+    // Every load of these 64 keys and values is issued before the first is used.
+    // Lane `lane` owns key base + lane for the value rows; for the score tiles, row `col`
+    // of tile `kt` is key base + 16*kt + col.  Keys past the end repeat the last key.
+    const int my_key = (base + lane < k_end) ? base + lane : k_end - 1;
+    const int my_phys = table[my_key / page_size] * page_size + my_key % page_size;
+    bf16x8 kf[TILES][KSTEPS];
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      const bf16x8 kf = *reinterpret_cast<const bf16x8*>(krow + ks * 32 + grp * 8);
-      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], s, 0, 0, 0);
+    for (int kt = 0; kt < TILES; ++kt) {
+      const int phys = __shfl(my_phys, kt * 16 + col, PYLON_WAVE);
+      const uint16_t* krow = k_cache + (static_cast<size_t>(phys) * n_kv_heads + kvh) * HD;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) kf[kt][ks] = *reinterpret_cast<const bf16x8*>(krow + ks * 32 + grp * 8);
     }
-    // lane holds, for head `col`, the scores of keys base + 4*grp + r
-    float sv[4];
+    PackedElems<EPL> vv[AD_SUPER];
+#pragma unroll
+    for (int kk = 0; kk < AD_SUPER; ++kk) {
+      const int pk = __shfl(my_phys, kk, PYLON_WAVE);
+      const uint16_t* vrow = v_cache + (static_cast<size_t>(pk) * n_kv_heads + kvh) * HD;
+      vv[kk].load(vrow + lane * EPL);
+    }
+
+    floatx4 s[TILES];
+#pragma unroll
+    for (int kt = 0; kt < TILES; ++kt) {
+      s[kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks)
+        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kt][ks], qf[ks], s[kt], 0, 0, 0);
+    }
+    // lane holds, for head `col`, the scores of keys base + 16*kt + 4*grp + r
     float tile_max = -INFINITY;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const bool live = base + 4 * grp + r < k_end;
-      sv[r] = live ? s[r] * scale : -INFINITY;
-      tile_max = fmaxf(tile_max, sv[r]);
-    }
+    for (int kt = 0; kt < TILES; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const bool live = base + 16 * kt + 4 * grp + r < k_end;
+        s[kt][r] = live ? s[kt][r] * scale : -INFINITY;
+        tile_max = fmaxf(tile_max, s[kt][r]);
+      }
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, PYLON_WAVE));
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, PYLON_WAVE));
     const float m_new = fmaxf(m_run, tile_max);  // finite: key `base` is always live
     const float corr = expf(m_run - m_new);
     float tile_sum = 0.f;
+    __builtin_amdgcn_wave_barrier();  // the previous round's reads of p_tile come first
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float p = expf(sv[r] - m_new);  // exp(-inf) = 0 for keys past the end
-      tile_sum += p;
-      if (col < AD_MAX_GROUP) p_tile[4 * grp + r][col] = p;
-    }
+    for (int kt = 0; kt < TILES; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = expf(s[kt][r] - m_new);  // exp(-inf) = 0 for keys past the end
+        tile_sum += p;
+        if (col < GP) p_tile[16 * kt + 4 * grp + r][col] = p;
+      }
     tile_sum += __shfl_xor(tile_sum, 16, PYLON_WAVE);
     tile_sum += __shfl_xor(tile_sum, 32, PYLON_WAVE);
     l_run = l_run * corr + tile_sum;
     m_run = m_new;
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();  // p_tile is private to the wave: program order suffices
     // rescale what has been accumulated: the factor of head h sits in lane h
 #pragma unroll
-    for (int h = 0; h < AD_MAX_GROUP; ++h) {
-      if (h < group) {
-        const float c = __shfl(corr, h, PYLON_WAVE);
+    for (int h = 0; h < GP; ++h) {
+      const float c = __shfl(corr, h, PYLON_WAVE);
 #pragma unroll
-        for (int i = 0; i < EPL; ++i) acc[h][i] *= c;
+      for (int i = 0; i < EPL; ++i) acc[h][i] *= c;
+    }
+    // keys past the end weigh 0 and their value row is the (finite) last key's
+#pragma unroll
+    for (int kk = 0; kk < AD_SUPER; ++kk) {
+      float v[EPL];
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) v[i] = vv[kk].get(i);
+#pragma unroll
+      for (int h = 0; h < GP; ++h) {
+        const float p = p_tile[kk][h];
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) acc[h][i] = fmaf(p, v[i], acc[h][i]);
       }
     }
-    const int live_keys = (k_end - base < AD_TILE) ? k_end - base : AD_TILE;
-    for (int kk = 0; kk < live_keys; ++kk) {
-      const int pk = __shfl(phys, kk, PYLON_WAVE);
-      const uint16_t* vrow = v_cache + (static_cast<size_t>(pk) * n_kv_heads + kvh) * HD;
-      float vv[EPL];
-      load_bf16_elems<EPL>(vrow + lane * EPL, vv);
-#pragma unroll
-      for (int h = 0; h < AD_MAX_GROUP; ++h) {
-        if (h < group) {
-          const float p = p_tile[kk][h];
-#pragma unroll
-          for (int i = 0; i < EPL; ++i) acc[h][i] = fmaf(p, vv[i], acc[h][i]);
-        }
-      }
-    }
-    __syncthreads();
   }
 
-  // results: acc[h][i] is element lane*EPL + i of head h
-  if (n_splits == 1) {
+  // leave this wave's partial result in LDS: acc[h][i] is element lane*EPL + i of head h
 #pragma unroll
-    for (int h = 0; h < AD_MAX_GROUP; ++h) {
-      if (h < group) {
-        const float inv = 1.0f / __shfl(l_run, h, PYLON_WAVE);
-        uint16_t* orow = out + (static_cast<size_t>(t) * n_heads + kvh * group + h) * HD;
-        float o[EPL];
+  for (int h = 0; h < GP; ++h) {
+    float* arow = part_acc + (static_cast<size_t>(wave) * GP + h) * HD;
 #pragma unroll
-        for (int i = 0; i < EPL; ++i) o[i] = acc[h][i] * inv;
-        store_bf16_elems<EPL>(orow + lane * EPL, o);
-      }
+    for (int i = 0; i < EPL; ++i) arow[lane * EPL + i] = acc[h][i];
+    const float mh = __shfl(m_run, h, PYLON_WAVE), lh = __shfl(l_run, h, PYLON_WAVE);
+    if (lane == 0) {
+      part_ml[(wave * GP + h) * 2] = mh;
+      part_ml[(wave * GP + h) * 2 + 1] = lh;
     }
-  } else {
+  }
+  __syncthreads();
+  // wave h merges head h over all ranges, in the order of the ranges
+  for (int h = wave; h < group; h += n_waves) {
+    float m = -INFINITY;
+    for (int w = 0; w < n_waves; ++w) m = fmaxf(m, part_ml[(w * GP + h) * 2]);
+    float l = 0.f;
+    float o[EPL];
 #pragma unroll
-    for (int h = 0; h < AD_MAX_GROUP; ++h) {
-      if (h < group) {
-        const size_t item = (static_cast<size_t>(t) * n_heads + kvh * group + h) * n_splits + split;
-        float* arow = part_acc + item * HD;
+    for (int i = 0; i < EPL; ++i) o[i] = 0.f;
+    for (int w = 0; w < n_waves; ++w) {
+      const float lw = part_ml[(w * GP + h) * 2 + 1];
+      const float f = (lw == 0.f) ? 0.f : expf(part_ml[(w * GP + h) * 2] - m);  // an empty range
+      l += lw * f;
+      const float* arow = part_acc + (static_cast<size_t>(w) * GP + h) * HD;
 #pragma unroll
-        for (int i = 0; i < EPL; ++i) arow[lane * EPL + i] = acc[h][i];
-        const float mh = __shfl(m_run, h, PYLON_WAVE), lh = __shfl(l_run, h, PYLON_WAVE);
-        if (lane == 0) {
-          part_ml[item * 2] = mh;
-          part_ml[item * 2 + 1] = lh;
-        }
-      }
+      for (int i = 0; i < EPL; ++i) o[i] = fmaf(arow[lane * EPL + i], f, o[i]);
     }
+    const float inv = 1.0f / l;
+    uint16_t* orow = out + (static_cast<size_t>(t) * n_heads + kvh * group + h) * HD + lane * EPL;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) orow[i] = float_to_bf16_bits(o[i] * inv);
   }
 }
 
-// One wavefront per (token, head): combine the key ranges' partial results.
-template <int EPL>
-__global__ __launch_bounds__(PYLON_WAVE) void attention_merge_kernel(uint16_t* __restrict__ out,
-                                                                     const float* __restrict__ part_acc,
-                                                                     const float* __restrict__ part_ml,
-                                                                     int n_splits) {
-  constexpr int HD = EPL * 64;
-  const int lane = threadIdx.x;
-  const size_t item = blockIdx.x;
-  const float* ml = part_ml + item * n_splits * 2;
-  float m = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) m = fmaxf(m, ml[2 * s]);
-  float l = 0.f;
-  float acc[EPL];
-#pragma unroll
-  for (int i = 0; i < EPL; ++i) acc[i] = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float ls = ml[2 * s + 1];
-    if (ls == 0.f) continue;  // an empty range
-    const float f = expf(ml[2 * s] - m);
-    l += ls * f;
-    const float* arow = part_acc + (item * n_splits + s) * HD;
-#pragma unroll
-    for (int i = 0; i < EPL; ++i) acc[i] = fmaf(arow[lane * EPL + i], f, acc[i]);
-  }
-  const float inv = 1.0f / l;
-  uint16_t* orow = out + item * HD;
-  float o[EPL];
-#pragma unroll
-  for (int i = 0; i < EPL; ++i) o[i] = acc[i] * inv;
-  store_bf16_elems<EPL>(orow + lane * EPL, o);
+static size_t decode_lds_bytes(int n_waves, int gp, int head_dim) {
+  return sizeof(float) * (static_cast<size_t>(n_waves) * AD_SUPER * gp +
+                          static_cast<size_t>(n_waves) * gp * head_dim + static_cast<size_t>(n_waves) * gp * 2);
 }
 
 template <int EPL>
-static void launch_decode(void* out, float* part_acc, float* part_ml, const void* q, const void* k_cache,
-                          const void* v_cache, const int* block_table, int table_width,
-                          const int* tok_row, const int* positions, int tokens, int n_heads,
-                          int n_kv_heads, int page_size, int window, float scale, int n_splits,
-                          hipStream_t stream) {
-  dim3 grid(n_splits, n_kv_heads, tokens), block(PYLON_WAVE);
-  hipLaunchKernelGGL((attention_decode_kernel<EPL, EPL * 2>), grid, block, 0, stream, (uint16_t*)out,
-                     part_acc, part_ml, (const uint16_t*)q, (const uint16_t*)k_cache,
-                     (const uint16_t*)v_cache, block_table, table_width, tok_row, positions, n_heads,
-                     n_kv_heads, page_size, window, scale, n_splits);
-  if (n_splits > 1)
-    hipLaunchKernelGGL((attention_merge_kernel<EPL>), dim3(tokens * n_heads), block, 0, stream,
-                       (uint16_t*)out, part_acc, part_ml, n_splits);
+static int launch_decode(void* out, const void* q, const void* k_cache, const void* v_cache,
+                         const int* block_table, int table_width, const int* tok_row,
+                         const int* positions, int tokens, int n_heads, int n_kv_heads, int page_size,
+                         int window, float scale, int n_waves, hipStream_t stream) {
+  const int group = n_heads / n_kv_heads;
+  const int gp = group <= 1 ? 1 : group <= 2 ? 2 : group <= 4 ? 4 : group <= 8 ? 8 : 16;
+  // the partial results of all waves have to fit into 64 KB of LDS
+  while (n_waves > 1 && decode_lds_bytes(n_waves, gp, EPL * 64) > 65536) n_waves /= 2;
+  const size_t lds = decode_lds_bytes(n_waves, gp, EPL * 64);
+  dim3 grid(n_kv_heads, tokens), block(n_waves * PYLON_WAVE);
+#define LAUNCH(GP)                                                                                          \
+  hipLaunchKernelGGL((attention_decode_kernel<EPL, EPL * 2, GP>), grid, block, lds, stream, (uint16_t*)out, \
+                     (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_table,   \
+                     table_width, tok_row, positions, n_heads, n_kv_heads, page_size, window, scale)
+  switch (gp) {
+    case 1: LAUNCH(1); break;
+    case 2: LAUNCH(2); break;
+    case 4: LAUNCH(4); break;
+    case 8: LAUNCH(8); break;
+    default: LAUNCH(16); break;
+  }
+#undef LAUNCH
+  return 0;
 }
 
-// q, out: [tokens, n_heads, head_dim] bf16. part_acc: float [tokens*n_heads*n_splits*head_dim],
-// part_ml: float [tokens*n_heads*n_splits*2] (both unused when n_splits == 1).
-extern "C" int pylon_attention_decode(void* out, float* part_acc, float* part_ml, const void* q,
-                                      const void* k_cache, const void* v_cache, const int* block_table,
-                                      int table_width, const int* tok_row, const int* positions,
-                                      int tokens, int n_heads, int n_kv_heads, int head_dim,
-                                      int page_size, int window, float scale, int n_splits,
+// q, out: [tokens, n_heads, head_dim] bf16; n_waves (1, 2, 4, 8 or 16) wavefronts share
+// the keys of one (token, key/value head).
+extern "C" int pylon_attention_decode(void* out, const void* q, const void* k_cache, const void* v_cache,
+                                      const int* block_table, int table_width, const int* tok_row,
+                                      const int* positions, int tokens, int n_heads, int n_kv_heads,
+                                      int head_dim, int page_size, int window, float scale, int n_waves,
                                       hipStream_t stream) {
   PYLON_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "attention_decode: %d query heads cannot be grouped over %d key/value heads", n_heads,
@@ -251,13 +262,13 @@ extern "C" int pylon_attention_decode(void* out, float* part_acc, float* part_ml
   PYLON_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256,
                 "attention_decode: head_dim %d is not 64, 128 or 256", head_dim);
   PYLON_REQUIRE(page_size > 0 && table_width > 0 && window >= 0, "attention_decode: bad page size, width or window");
-  PYLON_REQUIRE(n_splits >= 1 && n_splits <= 64, "attention_decode: 1..64 key ranges");
-  PYLON_REQUIRE(n_splits == 1 || (part_acc && part_ml), "attention_decode: key ranges need partial buffers");
+  PYLON_REQUIRE(n_waves == 1 || n_waves == 2 || n_waves == 4 || n_waves == 8 || n_waves == 16,
+                "attention_decode: 1, 2, 4, 8 or 16 waves per (token, head), got %d", n_waves);
   PYLON_REQUIRE(tokens <= 65535 && n_kv_heads <= 65535, "attention_decode: too many tokens or heads for one launch");
   if (tokens == 0) return 0;
-#define GO(D)                                                                                           \
-  launch_decode<D>(out, part_acc, part_ml, q, k_cache, v_cache, block_table, table_width, tok_row,     \
-                   positions, tokens, n_heads, n_kv_heads, page_size, window, scale, n_splits, stream)
+#define GO(D)                                                                                      \
+  launch_decode<D>(out, q, k_cache, v_cache, block_table, table_width, tok_row, positions, tokens, \
+                   n_heads, n_kv_heads, page_size, window, scale, n_waves, stream)
   switch (head_dim / 64) {
     case 1: GO(1); break;
     case 2: GO(2); break;

@@ -50,36 +50,89 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, TX* x, const TD* __restrict
   const TD* dr = delta ? delta + static_cast<size_t>(r_in) * dim : nullptr;
   TO* yr = out + static_cast<size_t>(r_out) * dim;
 
-  constexpr int KEEP = 8;  // elements per thread held in registers
-  float held[KEEP];
+  // Fast path (float rows whose length is a multiple of 4 and fits the registers): every
+  // load of the row is a 16-byte load issued before anything is stored, so the row costs
+  // one trip to memory.
+  constexpr int VEC = 4;  // float4 chunks per thread
+  if (sizeof(TX) == 4 && sizeof(TD) == 4 && (dim & 3) == 0 && dim <= 4 * VEC * static_cast<int>(blockDim.x) &&
+      (delta_stride & 3) == 0) {
+    const int chunks = dim >> 2;
+    const float4* x4 = reinterpret_cast<const float4*>(xr);
+    const float4* w4 = reinterpret_cast<const float4*>(w);
+    float4 held[VEC], wt[VEC];
+#pragma unroll
+    for (int n = 0; n < VEC; ++n) {
+      const int c = threadIdx.x + n * blockDim.x;
+      held[n] = (c < chunks) ? x4[c] : float4{0.f, 0.f, 0.f, 0.f};
+      wt[n] = (c < chunks) ? w4[c] : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    if (dr) {
+      const float4* d4 = reinterpret_cast<const float4*>(dr);
+      const long long stride4 = delta_stride >> 2;
+      float4 d[VEC];
+#pragma unroll
+      for (int n = 0; n < VEC; ++n) {
+        const int c = threadIdx.x + n * blockDim.x;
+        d[n] = (c < chunks) ? d4[c] : float4{0.f, 0.f, 0.f, 0.f};
+      }
+      // partial sums of the previous matrix product are added in a fixed order
+      for (int p = 1; p < n_delta; ++p) {
+#pragma unroll
+        for (int n = 0; n < VEC; ++n) {
+          const int c = threadIdx.x + n * blockDim.x;
+          if (c < chunks) {
+            const float4 e = d4[c + p * stride4];
+            d[n].x += e.x; d[n].y += e.y; d[n].z += e.z; d[n].w += e.w;
+          }
+        }
+      }
+#pragma unroll
+      for (int n = 0; n < VEC; ++n) {
+        held[n].x += d[n].x; held[n].y += d[n].y; held[n].z += d[n].z; held[n].w += d[n].w;
+      }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int n = 0; n < VEC; ++n)
+      ss += held[n].x * held[n].x + held[n].y * held[n].y + held[n].z * held[n].z + held[n].w * held[n].w;
+    const float total = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(total / static_cast<float>(dim) + eps);
+#pragma unroll
+    for (int n = 0; n < VEC; ++n) {
+      const int c = threadIdx.x + n * blockDim.x;
+      if (c < chunks) {
+        if (dr && write_resid) reinterpret_cast<float4*>(xr)[c] = held[n];
+        const float y0 = (held[n].x * inv) * wt[n].x, y1 = (held[n].y * inv) * wt[n].y;
+        const float y2 = (held[n].z * inv) * wt[n].z, y3 = (held[n].w * inv) * wt[n].w;
+        TO* dst = yr + 4 * c;
+        dst[0] = from_float<TO>(y0);
+        dst[1] = from_float<TO>(y1);
+        dst[2] = from_float<TO>(y2);
+        dst[3] = from_float<TO>(y3);
+      }
+    }
+    return;
+  }
+
   float ss = 0.f;
-  int n = 0;
-  for (int i = threadIdx.x; i < dim; i += blockDim.x, ++n) {
+  for (int i = threadIdx.x; i < dim; i += blockDim.x) {
     float v = to_float(xr[i]);
     if (dr) {
-      // partial sums of the previous matrix product are added in a fixed order
       float d = to_float(dr[i]);
       for (int p = 1; p < n_delta; ++p) d += to_float(dr[i + p * delta_stride]);
       v += d;
       if (write_resid) xr[i] = from_float<TX>(v);
     }
-    if (n < KEEP) held[n] = v;
     ss += v * v;
   }
   const float total = block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(total / static_cast<float>(dim) + eps);
-  n = 0;
-  for (int i = threadIdx.x; i < dim; i += blockDim.x, ++n) {
-    float v;
-    if (n < KEEP) {
-      v = held[n];
-    } else {
-      v = to_float(xr[i]);
-      if (dr && !write_resid) {
-        float d = to_float(dr[i]);
-        for (int p = 1; p < n_delta; ++p) d += to_float(dr[i + p * delta_stride]);
-        v += d;
-      }
+  for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+    float v = to_float(xr[i]);
+    if (dr && !write_resid) {
+      float d = to_float(dr[i]);
+      for (int p = 1; p < n_delta; ++p) d += to_float(dr[i + p * delta_stride]);
+      v += d;
     }
     yr[i] = from_float<TO>((v * inv) * w[i]);
   }
@@ -89,7 +142,7 @@ template <typename TX, typename TD>
 static void launch_rmsnorm_out(void* out, int out_dtype, TX* x, const TD* delta, int n_delta,
                                long long delta_stride, const float* w, const int* row_idx, int rows,
                                int dim, float eps, int write_resid, hipStream_t stream) {
-  dim3 grid(rows), block(dim >= 2048 ? 512 : 256);
+  dim3 grid(rows), block(dim > 4096 ? 1024 : 256);
   if (out_dtype == PYLON_F32)
     hipLaunchKernelGGL((rmsnorm_kernel<TX, TD, float>), grid, block, 0, stream, (float*)out, x, delta,
                        n_delta, delta_stride, w, row_idx, dim, eps, write_resid);

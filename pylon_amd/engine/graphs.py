@@ -14,6 +14,7 @@ ranges that depends on the batch size only.
 """
 from __future__ import annotations
 
+import gc
 import logging
 from typing import Dict, Optional, Sequence as Seq, Tuple
 
@@ -25,8 +26,13 @@ logger = logging.getLogger("pylon")
 
 
 class DecodeGraphs:
-    def __init__(self, runner, *, max_batch: int, max_pages_per_request: int) -> None:
-        self.runner = runner
+    def __init__(self, model, manager, arena, *, max_batch: int, max_pages_per_request: int) -> None:
+        # The model, manager and arena are held directly, not through the runner that owns
+        # this object: no reference cycle, so graphs are destroyed when the runner goes,
+        # never by a garbage collection that happens to run inside a later capture.
+        self.model = model
+        self.manager = manager
+        self.arena = arena
         self.max_batch = max_batch
         self.width = max_pages_per_request
         self.pool = torch.cuda.graph_pool_handle()
@@ -42,7 +48,7 @@ class DecodeGraphs:
         rows = len(entries)
         if rows > self.max_batch or rows in self.failed:
             return False
-        page = self.runner.manager.page_size
+        page = self.manager.page_size
         for e in entries:
             if len(e.tokens) != 1 or list(e.want) != [0]:
                 return False
@@ -54,31 +60,38 @@ class DecodeGraphs:
         """Replay (capturing first if need be).  Returns None if this batch size has no
         graph; the caller then runs the step kernel by kernel.  The cache is reserved and
         committed here exactly as an ordinary step does."""
-        runner = self.runner
         rows = len(entries)
-        manager = runner.manager
+        manager, model, arena = self.manager, self.model, self.arena
         pairs = [(e.seq, 1) for e in entries]
         entry = self.captured.get(rows)
         if entry is None:
             _, size = plan_layout(rows, rows, rows, len(manager.groups), self.width)
-            block = torch.empty(size, dtype=torch.int32, device=runner.model.device)
-            ctx = build_step(entries, manager, runner.arena, vocab_size=runner.model.spec.vocab_size,
+            block = torch.empty(size, dtype=torch.int32, device=model.device)
+            ctx = build_step(entries, manager, arena, vocab_size=model.spec.vocab_size,
                              width=self.width, device_block=block, fixed_shapes=True)
+            # No garbage collection while the stream is capturing: a finalizer that frees a
+            # device object (an event, another graph) is not allowed there and aborts.
+            gc.collect()
+            gc_was_enabled = gc.isenabled()
+            gc.disable()
             try:
-                torch.cuda.synchronize(runner.model.device)
+                torch.cuda.synchronize(model.device)
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph, pool=self.pool):
-                    logits = runner.model.step(ctx)
+                    logits = model.step(ctx)
             except Exception:  # noqa: BLE001 - a failed capture leaves this size to eager steps
                 logger.exception("decode_graph_capture_failed batch_size=%s", rows)
                 self.failed.add(rows)
                 manager.cancel(pairs)
                 return None
+            finally:
+                if gc_was_enabled:
+                    gc.enable()
             self.captured[rows] = (graph, block, logits)
             graph.replay()  # capture records only; this runs the step
         else:
             graph, block, logits = entry
-            build_step(entries, manager, runner.arena, vocab_size=runner.model.spec.vocab_size,
+            build_step(entries, manager, arena, vocab_size=model.spec.vocab_size,
                        width=self.width, device_block=block, fixed_shapes=True)
             graph.replay()
         self.replays += 1

@@ -98,7 +98,8 @@ class Runner:
         page = self.manager.page_size
         limit = max_tokens_per_request or self.model.spec.max_positions or self.manager.capacity_tokens
         limit = min(limit, self.manager.capacity_tokens)
-        self.graphs = DecodeGraphs(self, max_batch=max_batch or self.manager.slots.max_slots,
+        self.graphs = DecodeGraphs(self.model, self.manager, self.arena,
+                                   max_batch=max_batch or self.manager.slots.max_slots,
                                    max_pages_per_request=-(-limit // page))
 
     def synchronize(self) -> None:
