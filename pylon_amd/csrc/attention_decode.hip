@@ -11,8 +11,9 @@
 //
 // Scores come from the 16x16x32 bf16 matrix instruction with 16 keys as rows and the
 // group's query heads as columns (unused columns are zero).  The weighted sum of values
-// runs on the vector units with each lane owning head_dim/64 consecutive output elements,
-// so values are read as whole contiguous rows.  Softmax statistics are float throughout.
+// runs on the vector units: a value row is read by head_dim/8 lanes, 16 bytes each, so one
+// load instruction fetches the rows of several keys; every lane accumulates its eight
+// elements over its keys and the lane groups are summed at the end.  Softmax statistics are float throughout.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -21,28 +22,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 #define AD_MAX_GROUP 16
 #define AD_TILE 16   // keys per score tile
 #define AD_SUPER 64  // keys whose loads are in flight together (four score tiles)
-#define AD_MAX_WAVES 16
-
-// EPL consecutive bfloat16 elements kept packed (two per register) until they are used.
-template <int EPL>
-struct PackedElems {
-  uint32_t raw[(EPL + 1) / 2];
-  __device__ __forceinline__ void load(const uint16_t* p) {
-    if (EPL == 1) {
-      raw[0] = *p;
-    } else if (EPL == 2) {
-      raw[0] = *reinterpret_cast<const uint32_t*>(p);
-    } else {
-      const uint2 four = *reinterpret_cast<const uint2*>(p);
-      raw[0] = four.x;
-      raw[(EPL + 1) / 2 - 1] = four.y;
-    }
-  }
-  __device__ __forceinline__ float get(int i) const {
-    const uint32_t word = raw[i / 2];
-    return (i & 1) ? __uint_as_float(word & 0xffff0000u) : __uint_as_float(word << 16);
-  }
-};
+#define AD_MAX_WAVES 8
 
 // EPL = head_dim / 64, KSTEPS = head_dim / 32, GP = heads per group rounded up to 1, 2, 4, 8, 16
 template <int EPL, int KSTEPS, int GP>
@@ -64,8 +44,12 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
   const int col = lane & 15, grp = lane >> 4;
   const int kvh = blockIdx.x, t = blockIdx.y;
   const int group = n_heads / n_kv_heads;
+  // When tok_row is null, token t uses row t of the block table.  Its first 64 entries are
+  // then fetched together with the position (one trip to memory instead of two); lane i
+  // keeps entry i.
+  const int* table = block_table + static_cast<size_t>(tok_row ? tok_row[t] : t) * table_width;
+  const int table_entry = (lane < table_width) ? table[lane] : 0;
   const int pos = positions[t];
-  const int* table = block_table + static_cast<size_t>(tok_row[t]) * table_width;
 
   // the keys of this wave
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
@@ -93,18 +77,24 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
   }
 
   float m_run = -INFINITY, l_run = 0.f;  // for head `col` (same in the 4 lanes that share it)
-  float acc[GP][EPL];                    // rows past `group` hold nothing of use
+  constexpr int LPK = HD / 8;             // lanes that share one key's value row
+  constexpr int KPI = PYLON_WAVE / LPK;   // keys per value load instruction
+  const int vkey = lane / LPK, vchunk = lane % LPK;
+  float acc[GP][8];  // elements vchunk*8 .. +7 over this lane's keys; rows past `group` unused
 #pragma unroll
   for (int h = 0; h < GP; ++h)
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) acc[h][i] = 0.f;
+    for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
 
   for (int base = k_begin; base < k_end; base += AD_SUPER) {
     // Every load of these 64 keys and values is issued before the first is used.
     // Lane `lane` owns key base + lane for the value rows; for the score tiles, row `col`
     // of tile `kt` is key base + 16*kt + col.  Keys past the end repeat the last key.
     const int my_key = (base + lane < k_end) ? base + lane : k_end - 1;
-    const int my_phys = table[my_key / page_size] * page_size + my_key % page_size;
+    const int my_page = my_key / page_size;
+    int page_id = __shfl(table_entry, my_page & (PYLON_WAVE - 1), PYLON_WAVE);
+    if (my_page >= PYLON_WAVE) page_id = table[my_page];
+    const int my_phys = page_id * page_size + my_key % page_size;
     bf16x8 kf[TILES][KSTEPS];
 #pragma unroll
     for (int kt = 0; kt < TILES; ++kt) {
@@ -113,12 +103,13 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) kf[kt][ks] = *reinterpret_cast<const bf16x8*>(krow + ks * 32 + grp * 8);
     }
-    PackedElems<EPL> vv[AD_SUPER];
+    // values: LPK lanes read one key's row, 8 elements each; KPI keys per load instruction
+    uint4 vv[AD_SUPER / KPI];
 #pragma unroll
-    for (int kk = 0; kk < AD_SUPER; ++kk) {
-      const int pk = __shfl(my_phys, kk, PYLON_WAVE);
+    for (int i = 0; i < AD_SUPER / KPI; ++i) {
+      const int pk = __shfl(my_phys, i * KPI + vkey, PYLON_WAVE);
       const uint16_t* vrow = v_cache + (static_cast<size_t>(pk) * n_kv_heads + kvh) * HD;
-      vv[kk].load(vrow + lane * EPL);
+      vv[i] = *reinterpret_cast<const uint4*>(vrow + vchunk * 8);
     }
 
     floatx4 s[TILES];
@@ -163,29 +154,42 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
     for (int h = 0; h < GP; ++h) {
       const float c = __shfl(corr, h, PYLON_WAVE);
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) acc[h][i] *= c;
+      for (int i = 0; i < 8; ++i) acc[h][i] *= c;
     }
     // keys past the end weigh 0 and their value row is the (finite) last key's
 #pragma unroll
-    for (int kk = 0; kk < AD_SUPER; ++kk) {
-      float v[EPL];
+    for (int i = 0; i < AD_SUPER / KPI; ++i) {
+      const uint32_t w[4] = {vv[i].x, vv[i].y, vv[i].z, vv[i].w};
+      float v[8];
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) v[i] = vv[kk].get(i);
+      for (int j = 0; j < 4; ++j) {
+        v[2 * j] = __uint_as_float(w[j] << 16);
+        v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+      }
 #pragma unroll
       for (int h = 0; h < GP; ++h) {
-        const float p = p_tile[kk][h];
+        const float p = p_tile[i * KPI + vkey][h];
 #pragma unroll
-        for (int i = 0; i < EPL; ++i) acc[h][i] = fmaf(p, v[i], acc[h][i]);
+        for (int j = 0; j < 8; ++j) acc[h][j] = fmaf(p, v[j], acc[h][j]);
       }
     }
   }
+  // sum over the lane groups that took different keys (a fixed tree of additions)
+#pragma unroll
+  for (int h = 0; h < GP; ++h)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int off = LPK; off < PYLON_WAVE; off <<= 1) acc[h][j] += __shfl_xor(acc[h][j], off, PYLON_WAVE);
 
-  // leave this wave's partial result in LDS: acc[h][i] is element lane*EPL + i of head h
+  // leave this wave's partial result in LDS: acc[h][j] is element vchunk*8 + j of head h
 #pragma unroll
   for (int h = 0; h < GP; ++h) {
     float* arow = part_acc + (static_cast<size_t>(wave) * GP + h) * HD;
+    if (vkey == 0) {
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) arow[lane * EPL + i] = acc[h][i];
+      for (int j = 0; j < 8; ++j) arow[vchunk * 8 + j] = acc[h][j];
+    }
     const float mh = __shfl(m_run, h, PYLON_WAVE), lh = __shfl(l_run, h, PYLON_WAVE);
     if (lane == 0) {
       part_ml[(wave * GP + h) * 2] = mh;
@@ -247,7 +251,7 @@ static int launch_decode(void* out, const void* q, const void* k_cache, const vo
   return 0;
 }
 
-// q, out: [tokens, n_heads, head_dim] bf16; n_waves (1, 2, 4, 8 or 16) wavefronts share
+// q, out: [tokens, n_heads, head_dim] bf16; n_waves (1, 2, 4 or 8) wavefronts share
 // the keys of one (token, key/value head).
 extern "C" int pylon_attention_decode(void* out, const void* q, const void* k_cache, const void* v_cache,
                                       const int* block_table, int table_width, const int* tok_row,
@@ -262,8 +266,8 @@ extern "C" int pylon_attention_decode(void* out, const void* q, const void* k_ca
   PYLON_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256,
                 "attention_decode: head_dim %d is not 64, 128 or 256", head_dim);
   PYLON_REQUIRE(page_size > 0 && table_width > 0 && window >= 0, "attention_decode: bad page size, width or window");
-  PYLON_REQUIRE(n_waves == 1 || n_waves == 2 || n_waves == 4 || n_waves == 8 || n_waves == 16,
-                "attention_decode: 1, 2, 4, 8 or 16 waves per (token, head), got %d", n_waves);
+  PYLON_REQUIRE(n_waves == 1 || n_waves == 2 || n_waves == 4 || n_waves == 8,
+                "attention_decode: 1, 2, 4 or 8 waves per (token, head), got %d", n_waves);
   PYLON_REQUIRE(tokens <= 65535 && n_kv_heads <= 65535, "attention_decode: too many tokens or heads for one launch");
   if (tokens == 0) return 0;
 #define GO(D)                                                                                      \

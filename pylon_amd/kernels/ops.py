@@ -217,11 +217,11 @@ def decode_attention_ok(q: torch.Tensor, k_cache: torch.Tensor) -> bool:
 
 
 def decode_splits(tokens: int, n_kv_heads: int, max_len: Optional[int]) -> int:
-    """Wavefronts (1, 2, 4, 8 or 16) that share the keys of one (token, key/value head):
+    """Wavefronts (1, 2, 4 or 8) that share the keys of one (token, key/value head):
     ranges of about 64 keys (one batch of loads per wave) while the launch stays within a
     few thousand waves.  Without a known length (graph capture) the count depends on the
     batch size only."""
-    waves = 16
+    waves = 8
     while waves > 1 and tokens * n_kv_heads * waves > 4096:
         waves //= 2
     if max_len is not None:
@@ -231,10 +231,12 @@ def decode_splits(tokens: int, n_kv_heads: int, max_len: Optional[int]) -> int:
 
 
 def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
-                     block_table: torch.Tensor, tok_row: torch.Tensor, positions: torch.Tensor, *,
+                     block_table: torch.Tensor, tok_row: Optional[torch.Tensor], positions: torch.Tensor, *,
                      page_size: int, window: Optional[int], scale: float, n_splits: int) -> torch.Tensor:
     """Paged attention of a few bfloat16 query tokens; ``n_splits`` wavefronts share the
-    keys of each (token, key/value head) and merge their partial results."""
+    keys of each (token, key/value head) and merge their partial results.  ``tok_row`` None
+    means token ``t`` uses row ``t`` of the block table (a decode-only step), which saves
+    the kernel one dependent trip to memory."""
     if q.dim() != 3 or not decode_attention_ok(q, k_cache):
         raise KernelError("attention_decode does not take this geometry")
     tokens, n_heads, head_dim = q.shape
@@ -245,8 +247,13 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         raise KernelError("attention_decode: q and the caches differ in dtype")
     if pages * page_size >= 2 ** 31:
         raise KernelError("attention_decode: the cache holds more slots than an int32 can index")
-    if tok_row.numel() != tokens or positions.numel() != tokens or block_table.dim() != 2:
-        raise KernelError("attention_decode: one row id and one position per token, and a 2-D table")
+    if positions.numel() != tokens or block_table.dim() != 2:
+        raise KernelError("attention_decode: one position per token and a 2-D table are required")
+    if tok_row is None:
+        if block_table.shape[0] < tokens:
+            raise KernelError("attention_decode: without row ids the table needs a row per token")
+    elif tok_row.numel() != tokens:
+        raise KernelError("attention_decode: one row id per token is required")
     out = torch.empty_like(q)
     _lib.call("pylon_attention_decode", _dev(out, "out"), _dev(q, "q"), _dev(k_cache, "k_cache"),
               _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],

@@ -61,8 +61,9 @@ class Attention(Part):
         )
         if ctx.decode_only and ops.decode_attention_ok(q, cache.k):
             splits = ops.decode_splits(tokens, spec.n_kv_heads, None if ctx.fixed_shapes else ctx.max_len)
+            # in a decode-only step token t is row t
             context = ops.attention_decode(
-                q, cache.k, cache.v, cache.block_table, ctx.tok_row, ctx.positions,
+                q, cache.k, cache.v, cache.block_table, None, ctx.positions,
                 page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits,
             )
         elif ops.prefill_attention_ok(q, cache.k):
