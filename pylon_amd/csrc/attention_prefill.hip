@@ -3,7 +3,7 @@
 //
 // A workgroup of four wavefronts takes one tile of consecutive tokens of one request and
 // one key/value head, together with all query heads of that head's group: a (token, head)
-// pair is one of up to 128 query rows, 32 per wave.  Keys and values are walked 64 at a
+// pair is one of up to 64 query rows, 16 per wave.  Keys and values are walked 64 at a
 // time.  The workgroup stages the 64 keys (row-major) and the 64 values (transposed, so
 // that a lane can read four consecutive keys of one element) in LDS.  Scores are computed
 // transposed (keys as rows, queries as columns): the result registers of a score tile then
@@ -16,8 +16,8 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 #define AP_BK 64       // keys per iteration
-#define AP_ROWS 128    // query rows per workgroup
-#define AP_QT 2        // 16-row query tiles per wave
+#define AP_ROWS 64     // query rows per workgroup
+#define AP_QT 1        // 16-row query tiles per wave
 #define AP_VSTRIDE 66  // keys per row of the transposed value tile (+2: spreads LDS banks)
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
@@ -76,6 +76,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     for (int dt = 0; dt < DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
+  const float scale_log2 = scale * 1.44269504088896340736f;
   const int kv_last = pos0 + ntok - 1;
   const int k_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
   for (int kb = (k_lo / AP_BK) * AP_BK; kb <= kv_last; kb += AP_BK) {
@@ -117,7 +118,9 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
       }
     }
 
-    // mask, running softmax, and the probabilities as row operands of the value product
+    // mask, running softmax, and the probabilities as row operands of the value product.
+    // Scores are scaled by scale*log2(e) so that the exponentials are single exp2
+    // instructions; the running maximum is kept in the same units.
     bf16x8 pa[AP_QT][AP_BK / 32];
 #pragma unroll
     for (int qt = 0; qt < AP_QT; ++qt) {
@@ -129,8 +132,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int key = kb + kt * 16 + 4 * grp + r;
-          const bool seen = key <= qp && key >= lo;
-          const float v = seen ? s[qt][kt][r] * scale : -INFINITY;
+          const float v = (key <= qp && key >= lo) ? s[qt][kt][r] * scale_log2 : -INFINITY;
           s[qt][kt][r] = v;
           tile_max = fmaxf(tile_max, v);
         }
@@ -138,14 +140,14 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
       tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, PYLON_WAVE));
       const float m_new = fmaxf(m_run[qt], tile_max);
       const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen no key yet
-      const float corr = __expf(m_run[qt] - m_use);
+      const float corr = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
       float tile_sum = 0.f;
       float p[AP_BK / 16][4];
 #pragma unroll
       for (int kt = 0; kt < AP_BK / 16; ++kt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          p[kt][r] = __expf(s[qt][kt][r] - m_use);
+          p[kt][r] = __builtin_amdgcn_exp2f(s[qt][kt][r] - m_use);
           tile_sum += p[kt][r];
         }
       tile_sum += __shfl_xor(tile_sum, 16, PYLON_WAVE);
@@ -210,7 +212,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 
 // tiles: [n_tiles, 4] = (index of the tile's first token in q/out, its token count, its row of
 // the block table, the position of its first token).  A tile holds consecutive tokens of one
-// request, at most floor(128 / group) of them.
+// request, at most floor(64 / group) of them.
 extern "C" int pylon_attention_prefill(void* out, const void* q, const void* k_cache, const void* v_cache,
                                        const int* block_table, int table_width, const int* tiles,
                                        int n_tiles, int n_heads, int n_kv_heads, int head_dim,

@@ -33,6 +33,25 @@ extern "C" int pylon_embed(float* out, const void* table, int table_dtype, const
   PYLON_LAUNCHED("embed");
 }
 
+// Four consecutive elements number 4c .. 4c+3 of a row, as floats.
+__device__ __forceinline__ float4 load4(const float* p, long long c) {
+  return reinterpret_cast<const float4*>(p)[c];
+}
+__device__ __forceinline__ float4 load4(const bf16_t* p, long long c) {
+  const uint2 raw = reinterpret_cast<const uint2*>(p)[c];
+  return float4{__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
+                __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u)};
+}
+__device__ __forceinline__ void store4(float* p, long long c, float a, float b, float d, float e) {
+  reinterpret_cast<float4*>(p)[c] = float4{a, b, d, e};
+}
+__device__ __forceinline__ void store4(bf16_t* p, long long c, float a, float b, float d, float e) {
+  uint2 raw;
+  raw.x = static_cast<uint32_t>(float_to_bf16_bits(a)) | (static_cast<uint32_t>(float_to_bf16_bits(b)) << 16);
+  raw.y = static_cast<uint32_t>(float_to_bf16_bits(d)) | (static_cast<uint32_t>(float_to_bf16_bits(e)) << 16);
+  reinterpret_cast<uint2*>(p)[c] = raw;
+}
+
 // ---- RMSNorm ----------------------------------------------------------------------
 // y = (x * 1/sqrt(mean(x^2) + eps)) * w, in float, rounded once on the store.
 // One workgroup per output row. `row_idx` (optional) picks the input row of each
@@ -54,7 +73,7 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, TX* x, const TD* __restrict
   // load of the row is a 16-byte load issued before anything is stored, so the row costs
   // one trip to memory.
   constexpr int VEC = 4;  // float4 chunks per thread
-  if (sizeof(TX) == 4 && sizeof(TD) == 4 && (dim & 3) == 0 && dim <= 4 * VEC * static_cast<int>(blockDim.x) &&
+  if (sizeof(TX) == 4 && (dim & 3) == 0 && dim <= 4 * VEC * static_cast<int>(blockDim.x) &&
       (delta_stride & 3) == 0) {
     const int chunks = dim >> 2;
     const float4* x4 = reinterpret_cast<const float4*>(xr);
@@ -67,13 +86,12 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, TX* x, const TD* __restrict
       wt[n] = (c < chunks) ? w4[c] : float4{0.f, 0.f, 0.f, 0.f};
     }
     if (dr) {
-      const float4* d4 = reinterpret_cast<const float4*>(dr);
       const long long stride4 = delta_stride >> 2;
       float4 d[VEC];
 #pragma unroll
       for (int n = 0; n < VEC; ++n) {
         const int c = threadIdx.x + n * blockDim.x;
-        d[n] = (c < chunks) ? d4[c] : float4{0.f, 0.f, 0.f, 0.f};
+        d[n] = (c < chunks) ? load4(dr, c) : float4{0.f, 0.f, 0.f, 0.f};
       }
       // partial sums of the previous matrix product are added in a fixed order
       for (int p = 1; p < n_delta; ++p) {
@@ -81,7 +99,7 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, TX* x, const TD* __restrict
         for (int n = 0; n < VEC; ++n) {
           const int c = threadIdx.x + n * blockDim.x;
           if (c < chunks) {
-            const float4 e = d4[c + p * stride4];
+            const float4 e = load4(dr, c + p * stride4);
             d[n].x += e.x; d[n].y += e.y; d[n].z += e.z; d[n].w += e.w;
           }
         }
@@ -104,11 +122,7 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, TX* x, const TD* __restrict
         if (dr && write_resid) reinterpret_cast<float4*>(xr)[c] = held[n];
         const float y0 = (held[n].x * inv) * wt[n].x, y1 = (held[n].y * inv) * wt[n].y;
         const float y2 = (held[n].z * inv) * wt[n].z, y3 = (held[n].w * inv) * wt[n].w;
-        TO* dst = yr + 4 * c;
-        dst[0] = from_float<TO>(y0);
-        dst[1] = from_float<TO>(y1);
-        dst[2] = from_float<TO>(y2);
-        dst[3] = from_float<TO>(y3);
+        store4(yr, c, y0, y1, y2, y3);
       }
     }
     return;
@@ -228,12 +242,45 @@ __global__ void silu_gate_kernel(T* __restrict__ out, const T* __restrict__ gu, 
   }
 }
 
+// bfloat16 rows whose length is a multiple of 8: eight elements (16 bytes) per thread.
+__global__ void silu_gate_bf16x8_kernel(uint4* __restrict__ out, const uint4* __restrict__ gu, int chunks,
+                                        size_t total) {
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (; i < total; i += step) {
+    const size_t t = i / chunks;
+    const size_t c = i - t * chunks;
+    const uint4 g = gu[t * 2 * chunks + c];
+    const uint4 u = gu[t * 2 * chunks + chunks + c];
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t r[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
+      const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
+      const float a0 = (g0 / (1.0f + expf(-g0))) * u0;
+      const float a1 = (g1 / (1.0f + expf(-g1))) * u1;
+      r[j] = static_cast<uint32_t>(float_to_bf16_bits(a0)) | (static_cast<uint32_t>(float_to_bf16_bits(a1)) << 16);
+    }
+    out[i] = uint4{r[0], r[1], r[2], r[3]};
+  }
+}
+
 extern "C" int pylon_silu_gate(void* out, const void* gate_up, int dtype, int tokens, int inter,
                                hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(dtype), "silu_gate: unknown dtype");
   PYLON_REQUIRE(tokens >= 0 && inter > 0, "silu_gate: bad sizes tokens=%d inter=%d", tokens, inter);
   const size_t total = static_cast<size_t>(tokens) * inter;
   if (total == 0) return 0;
+  if (dtype == PYLON_BF16 && inter % 8 == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
+      (reinterpret_cast<uintptr_t>(gate_up) & 15) == 0) {
+    const size_t chunks_total = total / 8;
+    size_t nblocks = (chunks_total + 255) / 256;
+    if (nblocks > 65535u * 16u) nblocks = 65535u * 16u;
+    hipLaunchKernelGGL(silu_gate_bf16x8_kernel, dim3((unsigned)nblocks), dim3(256), 0, stream, (uint4*)out,
+                       (const uint4*)gate_up, inter / 8, chunks_total);
+    PYLON_LAUNCHED("silu_gate");
+  }
   size_t blocks = (total + 255) / 256;
   if (blocks > 65535u * 16u) blocks = 65535u * 16u;
   dim3 grid((unsigned)blocks), block(256);

@@ -84,6 +84,107 @@ __global__ void qkv_prepare_kernel(T* __restrict__ q_out, T* __restrict__ k_cach
   }
 }
 
+// The same for head sizes that are multiples of 64 with the whole head rotated (or none of
+// it): a lane owns head_dim/64 consecutive elements, loads and stores them as one vector,
+// and finds its rotation partner (element i + head_dim/2) in lane + 32.  No LDS.
+template <typename T, int EPL>
+__global__ void qkv_prepare_wide_kernel(T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                        const T* __restrict__ qkv, long long row_stride,
+                                        const float* __restrict__ q_weight, const float* __restrict__ k_weight,
+                                        float eps, const float* __restrict__ inv_freq,
+                                        const int* __restrict__ positions, const int* __restrict__ slot_map,
+                                        long long items, int n_heads, int n_kv_heads, int heads_per_token) {
+  constexpr int HD = EPL * 64;
+  const int lane = threadIdx.x & (PYLON_WAVE - 1);
+  const int wave = threadIdx.x / PYLON_WAVE;
+  const long long item = static_cast<long long>(blockIdx.x) * QKV_WAVES + wave;
+  if (item >= items) return;
+  const int t = static_cast<int>(item / heads_per_token);
+  const int s = static_cast<int>(item - static_cast<long long>(t) * heads_per_token);
+  const T* row = qkv + static_cast<size_t>(t) * row_stride;
+  const T* src;
+  T* dst = nullptr;
+  const float* weight = nullptr;
+  bool rotate = false;
+  if (s < n_heads) {
+    src = row + static_cast<size_t>(s) * HD;
+    dst = q_out + (static_cast<size_t>(t) * n_heads + s) * HD;
+    weight = q_weight;
+    rotate = inv_freq != nullptr;
+  } else {
+    const int slot = slot_map[t];
+    const int j = (s - n_heads) % n_kv_heads;
+    const bool is_key = (s - n_heads) < n_kv_heads;
+    src = row + (static_cast<size_t>(n_heads) + (is_key ? 0 : n_kv_heads) + j) * HD;
+    if (slot >= 0) dst = (is_key ? k_cache : v_cache) + (static_cast<size_t>(slot) * n_kv_heads + j) * HD;
+    weight = is_key ? k_weight : nullptr;
+    rotate = is_key && inv_freq != nullptr;
+  }
+  float v[EPL];
+  if (sizeof(T) == 2) {
+    if (EPL == 1) {
+      v[0] = to_float(src[lane]);
+    } else if (EPL == 2) {
+      const uint32_t two = *reinterpret_cast<const uint32_t*>(src + lane * 2);
+      v[0] = __uint_as_float(two << 16);
+      v[EPL - 1] = __uint_as_float(two & 0xffff0000u);
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPL; e += 2) {
+        const uint32_t two = *reinterpret_cast<const uint32_t*>(src + lane * EPL + e);
+        v[e] = __uint_as_float(two << 16);
+        v[e + 1 < EPL ? e + 1 : e] = __uint_as_float(two & 0xffff0000u);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) v[e] = to_float(src[lane * EPL + e]);
+  }
+  if (weight != nullptr) {
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) ss += v[e] * v[e];
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(HD) + eps);
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) v[e] = (v[e] * inv) * weight[lane * EPL + e];
+  }
+  if (rotate) {
+    const float pos = static_cast<float>(positions[t]);
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      const float other = __shfl_xor(v[e], 32, PYLON_WAVE);
+      const int pair = (lane & 31) * EPL + e;  // index of the (i, i + HD/2) pair
+      const float angle = pos * inv_freq[pair];
+      const float c = cosf(angle), sn = sinf(angle);
+      v[e] = (lane < 32) ? v[e] * c - other * sn : v[e] * c + other * sn;
+    }
+  }
+  if (dst != nullptr) {
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) dst[lane * EPL + e] = from_float<T>(v[e]);
+  }
+}
+
+template <typename T>
+static bool launch_wide(T* q_out, T* k_cache, T* v_cache, const T* qkv, long long row_stride,
+                        const float* q_weight, const float* k_weight, float eps, const float* inv_freq,
+                        const int* positions, const int* slot_map, long long items, int n_heads,
+                        int n_kv_heads, int head_dim, int heads_per_token, dim3 grid, dim3 block,
+                        hipStream_t stream) {
+#define GO(EPL)                                                                                       \
+  hipLaunchKernelGGL((qkv_prepare_wide_kernel<T, EPL>), grid, block, 0, stream, q_out, k_cache,       \
+                     v_cache, qkv, row_stride, q_weight, k_weight, eps, inv_freq, positions, slot_map, \
+                     items, n_heads, n_kv_heads, heads_per_token)
+  switch (head_dim) {
+    case 64: GO(1); return true;
+    case 128: GO(2); return true;
+    case 256: GO(4); return true;
+    default: return false;
+  }
+#undef GO
+}
+
 // qkv: [tokens, row_stride] with q heads first, then (if store_kv) k heads, then v heads.
 // q_out: [tokens, n_heads, head_dim]. k_cache/v_cache: [slots, n_kv_heads, head_dim] where a
 // slot is page*page_size + offset; slot_map[t] < 0 stores nothing for token t.
@@ -111,6 +212,19 @@ extern "C" int pylon_qkv_prepare(void* q_out, void* k_cache, void* v_cache, cons
   PYLON_REQUIRE(blocks < (1ll << 31), "qkv_prepare: too many heads to process in one launch");
   dim3 grid((unsigned)blocks), block(QKV_WAVES * PYLON_WAVE);
   const size_t lds = sizeof(float) * QKV_WAVES * head_dim;
+  // whole-head rotation (or none) at head sizes 64/128/256 takes the vector form
+  if ((inv_freq == nullptr || rot_dim == head_dim) && row_stride % 2 == 0) {
+    bool done;
+    if (dtype == PYLON_F32)
+      done = launch_wide<float>((float*)q_out, (float*)k_cache, (float*)v_cache, (const float*)qkv, row_stride,
+                                q_weight, k_weight, eps, inv_freq, positions, slot_map, items, n_heads,
+                                n_kv_heads, head_dim, heads_per_token, grid, block, stream);
+    else
+      done = launch_wide<bf16_t>((bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, (const bf16_t*)qkv,
+                                 row_stride, q_weight, k_weight, eps, inv_freq, positions, slot_map, items,
+                                 n_heads, n_kv_heads, head_dim, heads_per_token, grid, block, stream);
+    if (done) PYLON_LAUNCHED("qkv_prepare");
+  }
   if (dtype == PYLON_F32)
     hipLaunchKernelGGL(qkv_prepare_kernel<float>, grid, block, lds, stream, (float*)q_out, (float*)k_cache,
                        (float*)v_cache, (const float*)qkv, row_stride, q_weight, k_weight, eps, inv_freq,

@@ -263,7 +263,7 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     return out
 
 
-PREFILL_ROWS = 128  # (token, head) query rows one workgroup of the prefill kernel takes
+PREFILL_ROWS = 64  # (token, head) query rows one workgroup of the prefill kernel takes
 
 
 def prefill_attention_ok(q: torch.Tensor, k_cache: torch.Tensor) -> bool:
