@@ -384,23 +384,58 @@ def test_attention_prefill(ops, geom):
     assert float((got.float() - ref.float()).abs().max()) <= 3e-2
 
 
-def test_attention_finds_one_far_key_among_hundreds(ops):
+@pytest.mark.parametrize("kernel", ["general_f32", "general_bf16", "decode", "prefill"])
+def test_attention_finds_one_far_key_among_hundreds(ops, kernel):
     # Random keys would hide a key that is skipped; here one far key matches the query
     # exactly and strongly, so the output must be (almost) that key's value.
+    dtype = torch.float32 if kernel == "general_f32" else torch.bfloat16
     nh, nkv, hd, page = 2, 1, 64, 16
     n = 777
-    for far in (0, 15, 16, 400, 776 - 64, 776):
-        kc = rnd((50, page, nkv, hd), 17) * 0.01
-        vc = rnd((50, page, nkv, hd), 18)
+    for far in (0, 15, 16, 400, 776 - 64, 775, 776):
+        kc = (rnd((50, page, nkv, hd), 17) * 0.01).to(dtype)
+        vc = rnd((50, page, nkv, hd), 18).to(dtype)
         table = torch.arange(49, -1, -1, dtype=torch.int32).reshape(1, 50)
-        q = rnd((1, nh, hd), 19)
+        q = rnd((1, nh, hd), 19).to(dtype)
         page_id, off = int(table[0, far // page]), far % page
-        kc[page_id, off, 0] = q[0, 0] * 4.0
-        got = ops.paged_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV),
-                                  torch.zeros(1, dtype=torch.int32, device=DEV),
-                                  torch.tensor([n - 1], dtype=torch.int32, device=DEV),
-                                  page_size=page, window=None, scale=1.0)
-        assert torch.allclose(got[0, 0].cpu(), vc[page_id, off, 0], atol=1e-3), far
+        kc[page_id, off, 0] = (q[0, 0].float() * 4.0).to(dtype)
+        row = torch.zeros(1, dtype=torch.int32, device=DEV)
+        pos = torch.tensor([n - 1], dtype=torch.int32, device=DEV)
+        args = (q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV))
+        if kernel == "decode":
+            got = ops.attention_decode(*args, row, pos, page_size=page, window=None, scale=1.0, n_splits=8)
+        elif kernel == "prefill":
+            tiles = torch.tensor([[0, 1, 0, n - 1]], dtype=torch.int32, device=DEV)
+            got = ops.attention_prefill(*args, tiles, page_size=page, window=None, scale=1.0)
+        else:
+            got = ops.paged_attention(*args, row, pos, page_size=page, window=None, scale=1.0)
+        assert torch.allclose(got[0, 0].float().cpu(), vc[page_id, off, 0].float(), atol=2e-2), (kernel, far)
+
+
+@pytest.mark.parametrize("kernel", ["general", "decode", "prefill"])
+def test_attention_window_edge_fast_kernels(ops, kernel):
+    # the key at distance `window` must be invisible, the one at distance window-1 visible
+    nh, nkv, hd, page, window = 1, 1, 64, 16, 37
+    dtype = torch.bfloat16
+    kc = torch.zeros((8, page, nkv, hd), dtype=dtype)
+    vc = rnd((8, page, nkv, hd), 20, dtype)
+    table = torch.arange(8, dtype=torch.int32).reshape(1, 8)
+    q = torch.ones((1, nh, hd), dtype=dtype)
+    pos = 100
+    row = torch.zeros(1, dtype=torch.int32, device=DEV)
+    p = torch.tensor([pos], dtype=torch.int32, device=DEV)
+    for key, visible in ((pos - window, False), (pos - window + 1, True)):
+        k2 = kc.clone()
+        k2[key // page, key % page, 0] = 1.0  # a key that dominates: score 64 against 0
+        args = (q.to(DEV), k2.to(DEV), vc.to(DEV), table.to(DEV))
+        if kernel == "decode":
+            got = ops.attention_decode(*args, row, p, page_size=page, window=window, scale=1.0, n_splits=2)
+        elif kernel == "prefill":
+            tiles = torch.tensor([[0, 1, 0, pos]], dtype=torch.int32, device=DEV)
+            got = ops.attention_prefill(*args, tiles, page_size=page, window=window, scale=1.0)
+        else:
+            got = ops.paged_attention(*args, row, p, page_size=page, window=window, scale=1.0)
+        hit = torch.allclose(got[0, 0].float().cpu(), vc[key // page, key % page, 0].float(), atol=2e-2)
+        assert hit == visible, (kernel, key)
 
 
 def test_attention_window_edge(ops):
