@@ -5,7 +5,8 @@ and uniform-random token ids, on one MI355X.
 
 A "step" is one decode step: one token for each of ``batch`` running requests through
 the step function, then greedy sampling on the device and the copy of the chosen ids to
-the host.  ``value`` is decoded tokens per second at the default batch of 8.  The same
+the host.  As in the engine's ticks, a step is queued before the host has read the ids of
+the step before it (they are fed back on the device), and every step's ids are read.  ``value`` is decoded tokens per second at the default batch of 8.  The same
 line carries the prefill of 2,048 tokens, the decode step's share of the HBM roofline,
 and decode rates at batch 1 and 64.
 """
@@ -86,35 +87,44 @@ def decode_run(runner, cfg, batch: int, steps: int, warmup: int, seed: int):
     import numpy as np
     import torch
 
-    from pylon_amd.engine import StepEntry
-    from pylon_amd.kernels import ops
+    from pylon_amd.engine import PENDING, StepEntry
+    from pylon_amd.sampling import Sampler, Sampling
 
+    sampler = Sampler(runner.model.device)
+    greedy = [(Sampling(temperature=0.0), 0)] * batch
     rng = np.random.default_rng(seed)
     seqs = [runner.open(f"b{batch}-{i}") for i in range(batch)]
     prompts = [rng.integers(0, cfg.vocab_size, PROMPT_LEN).tolist() for _ in range(batch)]
     # prompts in portions of up to 2048 tokens, as the scheduler would cut them
     per_step = max(1, PREFILL_TOKENS // PROMPT_LEN)
-    logits = []
     for lo in range(0, batch, per_step):
         part = list(range(lo, min(batch, lo + per_step)))
         out = runner.step([StepEntry(seqs[i], prompts[i], [PROMPT_LEN - 1]) for i in part])
-        logits.append(out)
-    tokens = ops.argmax(torch.cat(logits)).cpu().tolist()
+        sampler.launch(out, greedy[: len(part)], chosen=runner.chosen, place=runner.logit_slots).result()
 
-    def one_step(tokens):
-        out = runner.step([StepEntry(seqs[i], [tokens[i]], [0]) for i in range(batch)])
-        return ops.argmax(out).cpu().tolist()
+    entries = [StepEntry(seqs[i], [PENDING], [0]) for i in range(batch)]
+    produced = []
 
+    def one_step(before):
+        out = runner.step(entries)
+        draw = sampler.launch(out, greedy, chosen=runner.chosen, place=runner.logit_slots)
+        if before is not None:
+            produced.append(before.result())
+        return draw
+
+    draw = None
     for _ in range(warmup):
-        tokens = one_step(tokens)
+        draw = one_step(draw)
     torch.cuda.synchronize()
     context_sum = 0
     started = time.perf_counter()
     for _ in range(steps):
         context_sum += sum(s.length + 1 for s in seqs)
-        tokens = one_step(tokens)
+        draw = one_step(draw)
+    produced.append(draw.result())
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - started
+    assert len(produced) == warmup + steps and all(len(p) == batch for p in produced)
     for s in seqs:
         runner.close(s)
     return elapsed, context_sum / steps  # seconds, mean cached tokens read per step (all rows)

@@ -26,6 +26,9 @@ class PylonConfig:
     cuda_graphs: bool = False
     admit_skip: int = 4
     page_size: int = 256
+    # Queue the next step before the host has read the tokens of the running one (they are
+    # fed back on the device); stop tokens are then noticed one step late.
+    run_ahead: bool = True
     # Explicit pool size in pages; None sizes the pool from free device memory.
     num_pages: Optional[int] = None
 
@@ -77,6 +80,7 @@ def get_config(**overrides) -> PylonConfig:
         batch_wait_ms=float(os.getenv("PYLON_BATCH_WAIT_MS", "2")),
         cuda_graphs=_env_bool("PYLON_CUDA_GRAPHS", False),
         admit_skip=int(os.getenv("PYLON_ADMIT_SKIP", "4")),
+        run_ahead=_env_bool("PYLON_RUN_AHEAD", True),
         page_size=int(os.getenv("PYLON_PAGE_SIZE", "256")),
         num_pages=int(num_pages) if num_pages else None,
     )

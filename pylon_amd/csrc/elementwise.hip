@@ -5,11 +5,15 @@
 
 // ---- embedding ------------------------------------------------------------------
 // out[t, :] = table[ids[t], :] * scale, written as float (the residual stream).
+// A negative id -(1 + s) stands for "the token that the sampler left in chosen[s]": a
+// request's last sampled token can be fed back without a trip through the host.
 template <typename T>
 __global__ void embed_kernel(float* __restrict__ out, const T* __restrict__ table,
-                             const int* __restrict__ ids, int hidden, int vocab, float scale) {
+                             const int* __restrict__ ids, const int* __restrict__ chosen, int hidden,
+                             int vocab, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
+  if (id < 0 && chosen != nullptr) id = chosen[-1 - id];
   // The host checks ids; the clamp only keeps a bad id from reading outside the table.
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const T* row = table + static_cast<size_t>(id) * hidden;
@@ -17,8 +21,11 @@ __global__ void embed_kernel(float* __restrict__ out, const T* __restrict__ tabl
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(row[i]) * scale;
 }
 
+// chosen may be null; then every id must be a table row.  The host guarantees that a
+// negative id -(1 + s) names an entry s inside chosen.
 extern "C" int pylon_embed(float* out, const void* table, int table_dtype, const int* ids,
-                           int tokens, int hidden, int vocab, float scale, hipStream_t stream) {
+                           const int* chosen, int tokens, int hidden, int vocab, float scale,
+                           hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(table_dtype), "embed: unknown table dtype %d", table_dtype);
   PYLON_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "embed: bad sizes tokens=%d hidden=%d vocab=%d",
                 tokens, hidden, vocab);
@@ -26,10 +33,10 @@ extern "C" int pylon_embed(float* out, const void* table, int table_dtype, const
   dim3 grid(tokens), block(256);
   if (table_dtype == PYLON_F32)
     hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, out, (const float*)table, ids,
-                       hidden, vocab, scale);
+                       chosen, hidden, vocab, scale);
   else
     hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, out, (const bf16_t*)table, ids,
-                       hidden, vocab, scale);
+                       chosen, hidden, vocab, scale);
   PYLON_LAUNCHED("embed");
 }
 

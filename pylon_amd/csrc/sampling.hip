@@ -47,28 +47,40 @@ __device__ int block_argmax(const float* __restrict__ row, int vocab, ArgBest* s
   return total.index;
 }
 
+// The chosen id goes to out[row] and, if asked for, also to chosen[place[row]]: a table
+// with one entry per request from which the next step's embedding can take its token.
+__device__ __forceinline__ void emit(int* __restrict__ out, int* __restrict__ chosen,
+                                     const int* __restrict__ place, int row, int id) {
+  out[row] = id;
+  if (chosen != nullptr) chosen[place[row]] = id;
+}
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void argmax_kernel(int* __restrict__ out,
                                                                 const float* __restrict__ logits,
-                                                                int vocab, long long row_stride) {
+                                                                int vocab, long long row_stride,
+                                                                int* __restrict__ chosen,
+                                                                const int* __restrict__ place) {
   __shared__ ArgBest scratch[16];
   const float* row = logits + static_cast<size_t>(blockIdx.x) * row_stride;
   const int idx = block_argmax(row, vocab, scratch);
-  if (threadIdx.x == 0) out[blockIdx.x] = idx;
+  if (threadIdx.x == 0) emit(out, chosen, place, blockIdx.x, idx);
 }
 
+// chosen and place are both null or both given (place: one index into chosen per row).
 extern "C" int pylon_argmax(int* out, const float* logits, int rows, int vocab, long long row_stride,
-                            hipStream_t stream) {
+                            int* chosen, const int* place, hipStream_t stream) {
+  PYLON_REQUIRE((chosen == nullptr) == (place == nullptr), "argmax: chosen and place go together");
   PYLON_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "argmax: bad sizes rows=%d vocab=%d", rows, vocab);
   if (rows == 0) return 0;
   hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, out, logits, vocab,
-                     row_stride);
+                     row_stride, chosen, place);
   PYLON_LAUNCHED("argmax");
 }
 
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     int* __restrict__ out, const float* __restrict__ logits, int vocab, long long row_stride,
     const float* __restrict__ temperature, const float* __restrict__ top_p,
-    const float* __restrict__ uniform) {
+    const float* __restrict__ uniform, int* __restrict__ chosen, const int* __restrict__ place) {
   __shared__ ArgBest best_scratch[16];
   __shared__ float scratch[16];
   __shared__ float wave_totals[16];
@@ -78,7 +90,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const float temp = temperature[r];
   if (temp <= 0.f) {
     const int idx = block_argmax(row, vocab, best_scratch);
-    if (threadIdx.x == 0) out[r] = idx;
+    if (threadIdx.x == 0) emit(out, chosen, place, r, idx);
     return;
   }
   const float inv_temp = 1.0f / temp;
@@ -162,20 +174,21 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     if (threadIdx.x == 0) {
       int v = -1;
       for (int wv = 0; wv < nwaves; ++wv) v = max(v, last_scratch[wv]);
-      out[r] = v < 0 ? 0 : v;
+      emit(out, chosen, place, r, v < 0 ? 0 : v);
     }
   } else if (threadIdx.x == 0) {
-    out[r] = found;
+    emit(out, chosen, place, r, found);
   }
 }
 
 extern "C" int pylon_sample(int* out, const float* logits, int rows, int vocab, long long row_stride,
                             const float* temperature, const float* top_p, const float* uniform,
-                            hipStream_t stream) {
+                            int* chosen, const int* place, hipStream_t stream) {
+  PYLON_REQUIRE((chosen == nullptr) == (place == nullptr), "sample: chosen and place go together");
   PYLON_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
   PYLON_REQUIRE(temperature && top_p && uniform, "sample: temperature, top_p and uniform are required");
   if (rows == 0) return 0;
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, out, logits, vocab,
-                     row_stride, temperature, top_p, uniform);
+                     row_stride, temperature, top_p, uniform, chosen, place);
   PYLON_LAUNCHED("sample");
 }

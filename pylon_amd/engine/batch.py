@@ -20,12 +20,17 @@ import torch
 from ..cache.manager import CacheManager, CacheView, Sequence
 
 
+#: In place of a token id: "the token that the sampler chose for this request last, and
+#: left on the device".  It lets a step be queued before the host has read that token.
+PENDING = -1
+
+
 @dataclass
 class StepEntry:
     """One request's share of a step: its next tokens and which of them need logits."""
 
     seq: Sequence
-    tokens: Seq[int]
+    tokens: Seq[int]  # token ids; PENDING where the id is still on the device
     want: Seq[int] = ()  # indices into `tokens`
 
 
@@ -99,6 +104,8 @@ class StepContext:
     max_len: int = 0
     decode_only: bool = False
     fixed_shapes: bool = False  # launches must not depend on lengths (graph capture)
+    logit_slots: Optional[torch.Tensor] = None  # int32 [n]: state slot of each wanted row's request
+    chosen: Optional[torch.Tensor] = None  # int32 [slots]: last sampled token per state slot
     _tiles: Dict[int, torch.Tensor] = field(default_factory=dict)
 
     def cache(self, cache_id: int) -> CacheView:
@@ -145,6 +152,7 @@ def plan_layout(tokens: int, rows: int, n_logits: int, n_groups: int, width: int
     put("row_slots", rows)
     put("row_first", rows)
     put("logit_idx", n_logits)
+    put("logit_slots", n_logits)
     for g in range(n_groups):
         put(f"slot_map{g}", tokens)
         put(f"block_table{g}", rows * width)
@@ -153,10 +161,13 @@ def plan_layout(tokens: int, rows: int, n_logits: int, n_groups: int, width: int
 
 def build_step(entries: Seq[StepEntry], manager: CacheManager, arena: MetadataArena, *,
                vocab_size: int, width: Optional[int] = None,
-               device_block: Optional[torch.Tensor] = None, fixed_shapes: bool = False) -> StepContext:
+               device_block: Optional[torch.Tensor] = None, fixed_shapes: bool = False,
+               chosen: Optional[torch.Tensor] = None) -> StepContext:
     """Check the entries, take the pages they need, and put the step's metadata on the
     device.  Raises before touching the cache if any entry is malformed; raises
-    :class:`~pylon_amd.cache.pages.OutOfPages` (cache untouched) if pages run short."""
+    :class:`~pylon_amd.cache.pages.OutOfPages` (cache untouched) if pages run short.
+    ``chosen`` is the table of last sampled tokens by state slot; only with it may an
+    entry hold :data:`PENDING`."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     rows = len(entries)
@@ -165,7 +176,10 @@ def build_step(entries: Seq[StepEntry], manager: CacheManager, arena: MetadataAr
         raise ValueError("Each packed sequence needs at least one query token.")
     tokens = int(counts.sum())
     flat = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
-    if flat.size and (flat.min() < 0 or flat.max() >= vocab_size):
+    pending = flat == PENDING
+    if pending.any() and chosen is None:
+        raise ValueError("A token left on the device needs the table of sampled tokens.")
+    if flat.size and (flat[~pending].min(initial=0) < 0 or flat.max() >= vocab_size):
         raise ValueError(f"Token IDs must be between 0 and {vocab_size - 1:,}.")
     row_start = np.zeros(rows + 1, dtype=np.int64)
     np.cumsum(counts, out=row_start[1:])
@@ -198,6 +212,9 @@ def build_step(entries: Seq[StepEntry], manager: CacheManager, arena: MetadataAr
         off, n = layout[name]
         return host[off: off + n]
 
+    token_slots = slots[tok_row]
+    if pending.any():
+        flat = np.where(pending, -1 - token_slots, flat)  # the embedding reads chosen[slot]
     seg("token_ids")[:] = flat
     seg("positions")[:] = positions
     seg("tok_row")[:] = tok_row
@@ -207,7 +224,7 @@ def build_step(entries: Seq[StepEntry], manager: CacheManager, arena: MetadataAr
     seg("row_first")[:] = starts == 0
     if logit_list:
         seg("logit_idx")[:] = logit_list
-    token_slots = slots[tok_row]
+        seg("logit_slots")[:] = token_slots[logit_list]
     for g in range(n_groups):
         manager.slot_map(g, token_slots, positions, seg(f"slot_map{g}"))
         manager.block_table(g, slots, width, seg(f"block_table{g}").reshape(rows, width))
@@ -230,6 +247,7 @@ def build_step(entries: Seq[StepEntry], manager: CacheManager, arena: MetadataAr
         row_start=dev("row_start"), seq_lens=dev("seq_lens"), row_slots=dev("row_slots"),
         row_first=dev("row_first"),
         logit_idx=dev("logit_idx") if logit_list else None, n_logits=len(logit_list),
+        logit_slots=dev("logit_slots") if logit_list else None, chosen=chosen,
         views=views, counts=counts, starts=starts, max_count=int(counts.max()),
         max_len=int(seq_lens.max()), decode_only=bool((counts == 1).all()),
         fixed_shapes=fixed_shapes,

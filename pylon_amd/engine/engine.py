@@ -7,6 +7,13 @@ A tick is the reference's (/root/reference/src/pylon/engine.py:255-300): drop ca
 requests, admit, run one step that carries every decoding request's pending token beside
 the prompt portions the token budget allows, sample where a row is ready, finish or
 continue each request, admit again into what was freed.
+
+Running ahead (``PylonConfig.run_ahead``, when the step executor keeps the sampler's last
+token of each request on the device): a tick queues its step and its sampling and only
+then reads the tokens of the tick before, so the device never waits for the host.  A
+decoding request's token is fed from the device (:data:`~pylon_amd.engine.batch.PENDING`).
+A request that meets a stop token has then already been given one more step; that step's
+token is dropped.  The end by ``max_new_tokens`` is known beforehand and costs nothing.
 """
 from __future__ import annotations
 
@@ -21,7 +28,7 @@ from typing import Callable, Deque, Iterable, List, Optional, Sequence, Tuple
 from ..cache.pages import OutOfPages
 from ..config.engine_config import PylonConfig
 from ..sampling.params import Sampling
-from .batch import StepEntry
+from .batch import PENDING, StepEntry
 from .scheduler import AdmissionPolicy, PromptWork, Waiter, cut_prompts, hold_prompts
 
 logger = logging.getLogger("pylon")
@@ -58,6 +65,17 @@ class Request:
 
 
 @dataclass
+class Flight:
+    """A queued step whose sampled tokens have not been read yet."""
+
+    draw: object  # .result() -> token ids of `ready`, in order
+    ready: List["Active"]
+    decoding: List["Active"]
+    portions: List[Tuple["Active", int]]
+    started: float
+
+
+@dataclass
 class Ticket:
     """A request waiting for admission."""
 
@@ -81,10 +99,19 @@ class Active:
     inter_token_seconds: List[float] = field(default_factory=list)
     prompt_wait_started: float = 0.0
     first_token_at: Optional[float] = None
+    # Running ahead: a sampled token waits on the device to be fed / how many sampled
+    # tokens the host has not read yet / the request has ended.
+    awaiting: bool = False
+    unread: int = 0
+    done: bool = False
 
     @property
     def request(self) -> Request:
         return self.ticket.request
+
+    @property
+    def decoding(self) -> bool:
+        return self.pending_token_id is not None or self.awaiting
 
     @property
     def remaining_prompt(self) -> int:
@@ -120,6 +147,10 @@ class Engine:
         manager = runner.manager
         self.page_size = manager.page_size
         self.kv_budget_pages = manager.num_pages
+        self._run_ahead = bool(config.run_ahead and hasattr(runner, "chosen")
+                               and hasattr(sampler, "launch"))
+        self._flight: Optional[Flight] = None
+        self._landed_at = 0.0
         self._policy = AdmissionPolicy(page_budget=manager.num_pages, page_size=manager.page_size,
                                        admit_skip=config.admit_skip)
         self._max_batch_size = config.max_batch_size
@@ -198,6 +229,7 @@ class Engine:
             self._closed = True
             waiting, self._waiting = list(self._waiting), deque()
             active, self._active = self._active, []
+            self._flight = None
             self._wake.notify_all()
         error = EngineClosedError("The generation scheduler is closed.")
         for item in active:
@@ -235,14 +267,18 @@ class Engine:
                 return False
             self._drop_cancelled_active()
             self._admit()
-            if self._active:
-                try:
-                    self._run_step()
-                except Exception as error:
-                    logger.exception("model_batch_failed")
-                    self._fail_active(error)
+            try:
+                flight = self._launch_step() if self._active else None
+                if self._run_ahead:
+                    # The step just queued runs behind the one before it; now read that one.
+                    flight, self._flight = self._flight, flight
+                if flight is not None:
+                    self._land(flight)
+            except Exception as error:
+                logger.exception("model_batch_failed")
+                self._fail_active(error)
             self._admit()
-            return bool(self._active or self._waiting)
+            return bool(self._active or self._waiting or self._flight)
 
     # ---- admission ----------------------------------------------------------------------------
     def _sweep_cancelled_waiting(self) -> None:
@@ -258,7 +294,7 @@ class Engine:
                 Waiter(t, len(t.request.input_ids) + t.request.sampling.max_new_tokens, t.arrived)
                 for t in self._waiting
             ]
-            decoding = sum(1 for a in self._active if a.pending_token_id is not None)
+            decoding = sum(1 for a in self._active if a.decoding)
             verdict = self._policy.next(waiters, reserved_pages=self.reserved_pages(),
                                         decoding=decoding, now=self._clock())
             if verdict is None:
@@ -294,11 +330,14 @@ class Engine:
         return True
 
     # ---- the step -----------------------------------------------------------------------------
-    def _run_step(self) -> None:
+    def _launch_step(self) -> Optional[Flight]:
+        """Queue one step and the sampling of its ready rows."""
         now = self._clock()
-        decoding = [a for a in self._active if a.pending_token_id is not None]
+        # A request whose unread tokens complete its max_new_tokens gets no further step.
+        decoding = [a for a in self._active if a.decoding
+                    and len(a.output_ids) + a.unread < a.request.sampling.max_new_tokens]
         work = [PromptWork(a, a.remaining_prompt, a.prompt_wait_started)
-                for a in self._active if a.pending_token_id is None and a.remaining_prompt > 0]
+                for a in self._active if not a.decoding and a.remaining_prompt > 0]
         portions: List[Tuple[Active, int]] = []
         if not hold_prompts(len(decoding), self._max_batch_size, work, now):
             portions = cut_prompts(work, self._prefill_chunk_size, now)
@@ -307,7 +346,8 @@ class Engine:
         entries: List[StepEntry] = []
         ready: List[Active] = []
         for item in decoding:
-            entries.append(StepEntry(item.seq, [item.pending_token_id], [0]))
+            token = PENDING if item.awaiting else item.pending_token_id
+            entries.append(StepEntry(item.seq, [token], [0]))
             ready.append(item)
         for item, count in portions:
             chunk = item.request.input_ids[item.prompt_offset: item.prompt_offset + count]
@@ -316,7 +356,7 @@ class Engine:
             if finishes:
                 ready.append(item)
         if not entries:
-            return
+            return None
         self.last_step = ([a.request.request_id for a in decoding],
                           [(a.request.request_id, c) for a, c in portions])
         started = self._clock()
@@ -325,24 +365,42 @@ class Engine:
         for item, count in portions:
             item.prompt_offset += count
             item.prompt_wait_started = self._clock()
-        token_ids: List[int] = []
-        if ready:
-            token_ids = self.sampler.sample(
-                logits, [(a.request.sampling, len(a.output_ids)) for a in ready]
-            )
-        elif hasattr(self.runner, "synchronize"):
-            self.runner.synchronize()
-        sampled_at = self._clock()
-        elapsed = sampled_at - started
         for item in decoding:
+            item.pending_token_id = None
+            item.awaiting = False
+        draw = None
+        if ready:
+            rows = [(a.request.sampling, len(a.output_ids) + a.unread) for a in ready]
+            if self._run_ahead:
+                draw = self.sampler.launch(logits, rows, chosen=self.runner.chosen,
+                                           place=self.runner.logit_slots)
+                for item in ready:
+                    item.awaiting = True
+            else:
+                draw = _Drawn(self.sampler.sample(logits, rows))
+            for item in ready:
+                item.unread += 1
+        elif not self._run_ahead and hasattr(self.runner, "synchronize"):
+            self.runner.synchronize()
+        return Flight(draw, ready, decoding, portions, started)
+
+    def _land(self, flight: Flight) -> None:
+        """Read a step's tokens; finish or continue its requests."""
+        token_ids = flight.draw.result() if flight.draw is not None else []
+        sampled_at = self._clock()
+        elapsed = sampled_at - max(flight.started, self._landed_at)
+        self._landed_at = sampled_at
+        for item in flight.decoding:
             item.inter_token_seconds.append(elapsed)
-        for item, _count in portions:
+        for item, _count in flight.portions:
             item.prefill_seconds += elapsed
-        finished = set()
-        for item, token_id in zip(ready, token_ids):
+        for item, token_id in zip(flight.ready, token_ids):
+            if item.done:
+                continue  # ended meanwhile (a stop token seen one step late, a cancellation)
+            item.unread -= 1
             if not self._accept(item, int(token_id), sampled_at):
-                finished.add(id(item))
-        self._active = [a for a in self._active if id(a) not in finished]
+                item.done = True
+        self._active = [a for a in self._active if not a.done]
 
     def _accept(self, item: Active, token_id: int, sampled_at: float) -> bool:
         """/root/reference/src/pylon/engine.py:598-618: a stop token ends the request and
@@ -356,7 +414,8 @@ class Engine:
         if len(item.output_ids) == item.request.sampling.max_new_tokens:
             self._complete(item, "length")
             return False
-        item.pending_token_id = token_id
+        if not self._run_ahead:
+            item.pending_token_id = token_id  # running ahead, the device feeds it
         return True
 
     def _complete(self, item: Active, reason: str) -> None:
@@ -375,6 +434,7 @@ class Engine:
         kept = []
         for item in self._active:
             if item.ticket.future.cancelled():
+                item.done = True
                 self.runner.close(item.seq)
             else:
                 kept.append(item)
@@ -384,10 +444,12 @@ class Engine:
         """A step that raised (pages ran short, a kernel refused) fails every running
         request and frees what they hold; waiting requests stay queued."""
         for item in self._active:
+            item.done = True
             self.runner.close(item.seq)
             if not item.ticket.future.done():
                 item.ticket.future.set_exception(error)
         self._active = []
+        self._flight = None
 
     # ---- validation ---------------------------------------------------------------------------
     def _validate_request(self, input_ids: List[int], stop_ids: frozenset, sampling: Sampling) -> None:
@@ -437,6 +499,16 @@ class Engine:
             except Exception as error:  # noqa: BLE001 - a broken tick fails what runs
                 with self._lock:
                     self._fail_active(error)
+
+
+class _Drawn:
+    """Token ids that are already on the host."""
+
+    def __init__(self, ids: List[int]) -> None:
+        self._ids = ids
+
+    def result(self) -> List[int]:
+        return self._ids
 
 
 def _load_runner(config: PylonConfig):

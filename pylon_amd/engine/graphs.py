@@ -26,17 +26,20 @@ logger = logging.getLogger("pylon")
 
 
 class DecodeGraphs:
-    def __init__(self, model, manager, arena, *, max_batch: int, max_pages_per_request: int) -> None:
+    def __init__(self, model, manager, arena, *, max_batch: int, max_pages_per_request: int,
+                 chosen: Optional[torch.Tensor] = None) -> None:
         # The model, manager and arena are held directly, not through the runner that owns
         # this object: no reference cycle, so graphs are destroyed when the runner goes,
         # never by a garbage collection that happens to run inside a later capture.
         self.model = model
         self.manager = manager
         self.arena = arena
+        self.chosen = chosen  # table of last sampled tokens, read by the recorded embedding
+        self.last_logit_slots: Optional[torch.Tensor] = None
         self.max_batch = max_batch
         self.width = max_pages_per_request
         self.pool = torch.cuda.graph_pool_handle()
-        self.captured: Dict[int, Tuple[torch.cuda.CUDAGraph, torch.Tensor, torch.Tensor]] = {}
+        self.captured: Dict[int, tuple] = {}
         self.failed = set()
         self.replays = 0
 
@@ -68,7 +71,8 @@ class DecodeGraphs:
             _, size = plan_layout(rows, rows, rows, len(manager.groups), self.width)
             block = torch.empty(size, dtype=torch.int32, device=model.device)
             ctx = build_step(entries, manager, arena, vocab_size=model.spec.vocab_size,
-                             width=self.width, device_block=block, fixed_shapes=True)
+                             width=self.width, device_block=block, fixed_shapes=True,
+                             chosen=self.chosen)
             # No garbage collection while the stream is capturing: a finalizer that frees a
             # device object (an event, another graph) is not allowed there and aborts.
             gc.collect()
@@ -87,12 +91,13 @@ class DecodeGraphs:
             finally:
                 if gc_was_enabled:
                     gc.enable()
-            self.captured[rows] = (graph, block, logits)
+            self.captured[rows] = (graph, block, logits, ctx.logit_slots)
+            self.last_logit_slots = ctx.logit_slots
             graph.replay()  # capture records only; this runs the step
         else:
-            graph, block, logits = entry
+            graph, block, logits, self.last_logit_slots = entry
             build_step(entries, manager, arena, vocab_size=model.spec.vocab_size,
-                       width=self.width, device_block=block, fixed_shapes=True)
+                       width=self.width, device_block=block, fixed_shapes=True, chosen=self.chosen)
             graph.replay()
         self.replays += 1
         manager.commit(pairs)

@@ -62,7 +62,8 @@ class Model(Part):
     def step(self, ctx: StepContext) -> Optional[torch.Tensor]:
         """Run the step's tokens through every scheduled layer, from and into the cache.
         Returns float32 logits ``[n_logits, vocab]`` (None when no logits are wanted)."""
-        resid = ops.embed(ctx.token_ids, self.params["embed"], scale=self.spec.embedding_scale)
+        resid = ops.embed(ctx.token_ids, self.params["embed"], scale=self.spec.embedding_scale,
+                          chosen=ctx.chosen)
         delta = None
         for layer, cache_id, stores in self.schedule:
             resid, delta = self.blocks[layer].forward(resid, delta, ctx, ctx.cache(cache_id), stores)

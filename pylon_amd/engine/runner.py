@@ -43,6 +43,10 @@ class Runner:
         )
         self.arena = MetadataArena(model.device)
         self.graphs = None
+        # Per-request state of the sampler, by state slot: the token chosen last.  A step
+        # may take a request's next token from here (StepEntry tokens = [PENDING]).
+        self.chosen = torch.zeros(self.manager.slots.max_slots, dtype=torch.int32, device=model.device)
+        self.logit_slots: Optional[torch.Tensor] = None  # state slot per row of the last step's logits
 
     # ---- construction ------------------------------------------------------------------
     @classmethod
@@ -100,7 +104,7 @@ class Runner:
         limit = min(limit, self.manager.capacity_tokens)
         self.graphs = DecodeGraphs(self.model, self.manager, self.arena,
                                    max_batch=max_batch or self.manager.slots.max_slots,
-                                   max_pages_per_request=-(-limit // page))
+                                   max_pages_per_request=-(-limit // page), chosen=self.chosen)
 
     def synchronize(self) -> None:
         torch.cuda.synchronize(self.model.device)
@@ -132,8 +136,11 @@ class Runner:
         if self.graphs is not None and self.graphs.wants(entries):
             logits = self.graphs.run(entries)
             if logits is not None:
+                self.logit_slots = self.graphs.last_logit_slots
                 return logits
-        ctx = build_step(entries, self.manager, self.arena, vocab_size=self.model.spec.vocab_size)
+        ctx = build_step(entries, self.manager, self.arena, vocab_size=self.model.spec.vocab_size,
+                         chosen=self.chosen)
+        self.logit_slots = ctx.logit_slots
         pairs = [(e.seq, len(e.tokens)) for e in entries]
         try:
             logits = self.model.step(ctx)

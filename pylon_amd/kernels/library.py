@@ -25,7 +25,7 @@ _lib_path: Optional[Path] = None
 P, I, F, L = c_void_p, c_int, c_float, c_longlong
 
 _SIGNATURES = {
-    "pylon_embed": [P, P, I, P, I, I, I, F, P],
+    "pylon_embed": [P, P, I, P, P, I, I, I, F, P],
     "pylon_rmsnorm": [P, I, P, I, P, P, I, I, F, P],
     "pylon_add_rmsnorm": [P, I, P, P, I, I, L, P, P, I, I, F, P],
     "pylon_residual_add": [P, P, I, L, P],
@@ -36,8 +36,8 @@ _SIGNATURES = {
     "pylon_attention_prefill": [P, P, P, P, P, I, P, I, I, I, I, I, I, F, P],
     "pylon_gemm_tiled": [P, I, P, I, P, I, I, I, I, L, L, L, P],
     "pylon_gemm_skinny": [P, I, P, P, I, I, I, L, L, L, I, L, I, P],
-    "pylon_argmax": [P, P, I, I, L, P],
-    "pylon_sample": [P, P, I, I, L, P, P, P, P],
+    "pylon_argmax": [P, P, I, I, L, P, P, P],
+    "pylon_sample": [P, P, I, I, L, P, P, P, P, P, P],
 }
 
 

@@ -42,8 +42,9 @@ def _dev(t: Optional[torch.Tensor], name: str, dtype=None) -> int:
 
 
 def embed(ids: torch.Tensor, table: torch.Tensor, *, scale: float = 1.0,
-          out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """float32 ``out[t] = table[ids[t]] * scale``."""
+          out: Optional[torch.Tensor] = None, chosen: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 ``out[t] = table[ids[t]] * scale``.  With ``chosen`` (int32, on the device) an
+    id ``-(1 + s)`` is replaced by ``chosen[s]``: the token a sampler left there."""
     tokens = ids.numel()
     vocab, hidden = table.shape
     if out is None:
@@ -51,7 +52,8 @@ def embed(ids: torch.Tensor, table: torch.Tensor, *, scale: float = 1.0,
     elif out.shape != (tokens, hidden):
         raise KernelError(f"embed: out has shape {tuple(out.shape)}, expected {(tokens, hidden)}")
     _lib.call("pylon_embed", _dev(out, "out", torch.float32), _dev(table, "table"),
-              dtype_code(table.dtype), _dev(ids, "ids", torch.int32), tokens, hidden, vocab,
+              dtype_code(table.dtype), _dev(ids, "ids", torch.int32),
+              None if chosen is None else _dev(chosen, "chosen", torch.int32), tokens, hidden, vocab,
               float(scale), _stream())
     return out
 
@@ -406,20 +408,46 @@ def linear_glu(x: torch.Tensor, gate_up: torch.Tensor, *, out_dtype: torch.dtype
     return silu_gate(linear(x, gate_up, out_dtype=out_dtype))
 
 
-def argmax(logits: torch.Tensor) -> torch.Tensor:
+def _chosen_args(rows: int, chosen: Optional[torch.Tensor], place: Optional[torch.Tensor]):
+    """The optional table that also receives the chosen ids: ``chosen[place[r]] = id``."""
+    if chosen is None and place is None:
+        return None, None
+    if chosen is None or place is None:
+        raise KernelError("chosen and place go together")
+    if place.numel() != rows:
+        raise KernelError("place must have one index per row")
+    return _dev(chosen, "chosen", torch.int32), _dev(place, "place", torch.int32)
+
+
+def _ids_out(rows: int, device, out: Optional[torch.Tensor]) -> torch.Tensor:
+    if out is None:
+        return torch.empty((rows,), dtype=torch.int32, device=device)
+    if out.shape != (rows,) or out.dtype != torch.int32 or not out.is_cuda:
+        raise KernelError("out must be int32 [rows] on the GPU")
+    return out
+
+
+def argmax(logits: torch.Tensor, *, out: Optional[torch.Tensor] = None,
+           chosen: Optional[torch.Tensor] = None, place: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The index of each row's largest logit (the lowest among equals); with ``chosen`` and
+    ``place`` the ids are also written to ``chosen[place[r]]``."""
     if logits.dim() != 2 or logits.stride(1) != 1:
         raise KernelError("argmax takes [rows, vocab] logits with contiguous rows")
     rows, vocab = logits.shape
-    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
     if not logits.is_cuda or logits.dtype != torch.float32:
         raise KernelError("argmax takes float32 logits on the GPU")
-    _lib.call("pylon_argmax", out.data_ptr(), logits.data_ptr(), rows, vocab, logits.stride(0), _stream())
+    out = _ids_out(rows, logits.device, out)
+    chosen_ptr, place_ptr = _chosen_args(rows, chosen, place)
+    _lib.call("pylon_argmax", out.data_ptr(), logits.data_ptr(), rows, vocab, logits.stride(0),
+              chosen_ptr, place_ptr, _stream())
     return out
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
-           uniform: torch.Tensor) -> torch.Tensor:
-    """One token per row; rows with temperature 0 take the argmax."""
+           uniform: torch.Tensor, *, out: Optional[torch.Tensor] = None,
+           chosen: Optional[torch.Tensor] = None, place: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token per row; rows with temperature 0 take the argmax.  ``chosen`` and ``place``
+    as for :func:`argmax`."""
     if logits.dim() != 2 or logits.stride(1) != 1:
         raise KernelError("sample takes [rows, vocab] logits with contiguous rows")
     rows, vocab = logits.shape
@@ -428,8 +456,9 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
     for name, t in (("temperature", temperature), ("top_p", top_p), ("uniform", uniform)):
         if t.numel() != rows:
             raise KernelError(f"sample: {name} must have one value per row")
-    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    out = _ids_out(rows, logits.device, out)
+    chosen_ptr, place_ptr = _chosen_args(rows, chosen, place)
     _lib.call("pylon_sample", out.data_ptr(), logits.data_ptr(), rows, vocab, logits.stride(0),
               _dev(temperature, "temperature", torch.float32), _dev(top_p, "top_p", torch.float32),
-              _dev(uniform, "uniform", torch.float32), _stream())
+              _dev(uniform, "uniform", torch.float32), chosen_ptr, place_ptr, _stream())
     return out

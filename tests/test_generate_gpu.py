@@ -147,3 +147,34 @@ def test_long_decoding_stays_on_the_plain_model(tmp):
     err = np.abs(got - want).max(axis=1)
     assert err.max() <= 2e-5 * np.abs(want).max(), int(err.argmax())
     assert len(set(tokens[len(prompt):])) > 3  # the model does not just repeat one token
+
+
+@pytest.mark.parametrize("graphs", [False, True])
+def test_running_ahead_gives_the_tokens_of_the_tick_by_tick_engine(tmp, graphs):
+    """The same requests (greedy and seeded sampling, with a stop token) with and without
+    the next step queued before the last one's tokens are read."""
+    from pylon_amd.engine.engine import Engine
+    from pylon_amd.sampling import Sampling
+
+    folder = make_model_folder(tmp, "A", dtype="bfloat16", std=0.08)
+    cfg, _ = read_folder(folder)
+    prompts = [random_tokens(cfg["vocab_size"], n, 30 + n) for n in (3, 9, 20, 41)]
+    outputs = []
+    for ahead in (False, True):
+        engine = Engine.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=24, max_batch_size=4,
+                                    prefill_chunk_size=16, run_ahead=ahead, cuda_graphs=graphs)
+        assert engine._run_ahead == ahead
+        try:
+            greedy = engine.generate(prompts, Sampling(max_new_tokens=40, temperature=0.0))
+            stop = greedy[1].output_ids[7]
+            cut = engine.generate(prompts, Sampling(max_new_tokens=40, temperature=0.0), eos_token_id=stop)
+            drawn = engine.generate(prompts, Sampling(max_new_tokens=40, temperature=0.9, top_p=0.9, seed=5))
+        finally:
+            engine.close()
+        assert engine.runner.manager.free_pages == 24
+        engine.runner.manager.check()
+        if graphs:
+            assert engine.runner.graphs.replays > 0
+        outputs.append([(r.output_ids, r.finish_reason) for r in greedy + cut + drawn])
+        assert any(reason == "eos" for _, reason in outputs[-1])
+    assert outputs[0] == outputs[1]

@@ -47,6 +47,34 @@ def test_embed(ops, dtype):
     assert np.array_equal(f64(out), f64(table)[ids.numpy()] * 0.5)
 
 
+def test_sampled_tokens_are_fed_back_on_the_device(ops):
+    """argmax / sample leave each row's id in chosen[place[row]]; the embedding takes an id
+    -(1 + s) from chosen[s]."""
+    vocab = 211
+    logits = rnd((3, vocab), 31) * 3
+    chosen = torch.full((6,), -7, dtype=torch.int32, device=DEV)
+    place = torch.tensor([4, 0, 5], dtype=torch.int32, device=DEV)
+    out = torch.empty(3, dtype=torch.int32, device=DEV)
+    got = ops.argmax(logits.to(DEV), out=out, chosen=chosen, place=place)
+    want = f64(logits).argmax(axis=1).tolist()
+    assert got.data_ptr() == out.data_ptr() and got.cpu().tolist() == want
+    assert chosen.cpu().tolist() == [want[1], -7, -7, -7, want[0], want[2]]
+    temps = torch.tensor([0.0, 0.7, 1.3], device=DEV)
+    u = torch.tensor([0.0, 0.3, 0.8], device=DEV)
+    plain_draw = ops.sample(logits.to(DEV), temps, torch.ones(3, device=DEV), u).cpu().tolist()
+    chosen.fill_(-7)
+    drawn = ops.sample(logits.to(DEV), temps, torch.ones(3, device=DEV), u, chosen=chosen, place=place)
+    assert drawn.cpu().tolist() == plain_draw
+    assert chosen.cpu().tolist() == [plain_draw[1], -7, -7, -7, plain_draw[0], plain_draw[2]]
+    table = rnd((vocab, 40), 32)
+    ids = torch.tensor([3, -1 - 4, -1 - 0, 9], dtype=torch.int32, device=DEV)
+    emb = ops.embed(ids, table.to(DEV), chosen=chosen)
+    rows = [3, plain_draw[0], plain_draw[1], 9]
+    assert np.array_equal(f64(emb), f64(table)[rows])
+    with pytest.raises(Exception):
+        ops.argmax(logits.to(DEV), chosen=chosen)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("dim", [80, 1000, 2560 + 16])
 def test_rmsnorm_and_fused_residual(ops, dtype, dim):

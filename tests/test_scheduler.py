@@ -384,3 +384,133 @@ def test_threaded_engine_serves_requests():
         assert [r.finish_reason for r in results] == ["length", "length"]
     finally:
         engine.close()
+
+
+# ---- running ahead: the next step is queued before the last one's tokens are read -----------
+
+class DeviceTableRunner(FakeRunner):
+    """A fake step function that also keeps the 'device' table of last sampled tokens: a
+    token given as PENDING is looked up there, as the embedding kernel does."""
+
+    def __init__(self, *args, **kw):
+        super().__init__(*args, **kw)
+        self.chosen = {}
+        self.logit_slots = None
+
+    def step(self, entries):
+        from pylon_amd.engine.batch import PENDING
+
+        ready = super().step(entries)
+        seen = []
+        for e, record in zip(entries, self.steps[-1]):
+            seen.append((record[0], [self.chosen[e.seq.slot] if t == PENDING else t for t in e.tokens],
+                         record[2], [t == PENDING for t in e.tokens]))
+        self.steps[-1] = seen
+        self.logit_slots = [e.seq.slot for e in entries if e.want]
+        return ready
+
+
+class LaggedSampler(ScriptedSampler):
+    """Writes the device table at once (stream order) but counts how often the host reads."""
+
+    def __init__(self):
+        super().__init__()
+        self.reads = 0
+
+    def launch(self, logits, rows, *, chosen, place):
+        ids = self.sample(logits, rows)
+        for slot, token in zip(place, ids):
+            chosen[slot] = token
+        sampler = self
+
+        class Draw:
+            def result(self):
+                sampler.reads += 1
+                return ids
+
+        return Draw()
+
+
+def make_ahead_engine(pages=8, slots=8, chunk=2048, **kw):
+    runner = DeviceTableRunner(pages, max_requests=slots, **kw)
+    clock = Clock()
+    config = PylonConfig(max_batch_size=slots, prefill_chunk_size=chunk, page_size=PAGE)
+    engine = Engine(config, runner=runner, sampler=LaggedSampler(), clock=clock)
+    assert engine._run_ahead
+    return engine, runner, clock
+
+
+def test_run_ahead_feeds_tokens_from_the_device_and_length_costs_no_extra_step():
+    engine, runner, _ = make_ahead_engine(chunk=4)
+    engine.sampler.scripts["a"] = [3, 4, 5]
+    future = enqueue(engine, "a", list(range(6)), 3)
+    engine.tick()  # portion of 4: nothing sampled
+    engine.tick()  # portion of 2, first token sampled, not read yet
+    assert engine.sampler.reads == 0 and len(runner.steps) == 2
+    engine.tick()  # decode step queued with the token still "on the device"; then token 0 read
+    assert runner.steps[2] == [("a", [3], [0], [True])]
+    assert engine.sampler.reads == 1
+    engine.run_until_idle()
+    # prompt in two portions + two decode steps: the third token ends the request by length,
+    # which is known beforehand, so no further step was queued
+    assert len(runner.steps) == 4
+    assert runner.steps[3] == [("a", [4], [0], [True])]
+    result = future.result(timeout=0)
+    assert result.output_ids == [3, 4, 5] and result.finish_reason == "length"
+    assert [call[0][1] for call in engine.sampler.calls] == [0, 1, 2]  # the draws' numbers
+    assert runner.manager.free_pages == 8 and not runner.manager.live_sequences()
+    runner.manager.check()
+
+
+def test_run_ahead_sees_a_stop_token_one_step_late_and_drops_that_step():
+    engine, runner, _ = make_ahead_engine()
+    engine.sampler.scripts["a"] = [3, 9, 6, 6]
+    engine.sampler.scripts["b"] = [1, 2, 3, 4]
+    fa = enqueue(engine, "a", [1, 2, 3], 8, eos=9)
+    fb = enqueue(engine, "b", [4, 5], 4)
+    engine.run_until_idle()
+    assert fa.result(timeout=0).output_ids == [3] and fa.result(timeout=0).finish_reason == "eos"
+    assert fb.result(timeout=0).output_ids == [1, 2, 3, 4]
+    # a was given exactly one step after the one that sampled its stop token
+    a_steps = [row for step in runner.steps for row in step if row[0] == "a"]
+    assert [tokens for _, tokens, _, _ in a_steps] == [[1, 2, 3], [3], [9]]
+    b_steps = [row for step in runner.steps for row in step if row[0] == "b"]
+    assert [tokens for _, tokens, _, _ in b_steps] == [[4, 5], [1], [2], [3]]
+    assert runner.manager.free_pages == 8 and not runner.manager.live_sequences()
+    runner.manager.check()
+
+
+def test_run_ahead_matches_the_tick_by_tick_engine():
+    scripts = {"a": [5, 6, 7, 9, 1], "b": [2, 2, 2, 2, 2, 2], "c": [9]}
+    outputs = []
+    for ahead in (False, True):
+        engine, runner, _ = (make_ahead_engine if ahead else make_engine)(chunk=4)
+        engine.sampler.scripts.update({k: list(v) for k, v in scripts.items()})
+        futures = [enqueue(engine, "a", list(range(9)), 6, eos=9), enqueue(engine, "b", [1], 5),
+                   enqueue(engine, "c", [3, 3], 3, eos=9)]
+        engine.run_until_idle()
+        outputs.append([(f.result(timeout=0).output_ids, f.result(timeout=0).finish_reason) for f in futures])
+        assert runner.manager.free_pages == 8
+    assert outputs[0] == outputs[1] == [([5, 6, 7], "eos"), ([2, 2, 2, 2, 2], "length"), ([], "eos")]
+
+
+def test_run_ahead_cancellation_and_failure_with_a_step_in_flight():
+    engine, runner, _ = make_ahead_engine()
+    fa = enqueue(engine, "a", [1, 2], 8)
+    fb = enqueue(engine, "b", [3], 8)
+    engine.tick()
+    engine.tick()  # a decode step is in flight
+    # cancel is refused for a running future; the engine's own cancellation path is the flag
+    fa.cancel()
+    runner.fail_next = OutOfPages("no free page")
+    engine.tick()
+    with pytest.raises(OutOfPages):
+        fb.result(timeout=0)
+    assert fa.done()
+    assert engine._flight is None and not ids(engine, "active")
+    assert runner.manager.free_pages == 8 and not runner.manager.live_sequences()
+    runner.manager.check()
+    # and the engine goes on
+    fc = enqueue(engine, "c", [1], 2)
+    engine.run_until_idle()
+    assert fc.result(timeout=0).output_ids == [7, 7]
