@@ -1,19 +1,47 @@
-// Choosing the next token from float logits, one workgroup per row:
+// Choosing the next token from float logits:
 //   temperature 0  -> the index of the largest logit (the lowest index among equals);
 //   temperature T  -> p = softmax(logits / T); with top_p < 1 only tokens whose
 //                     strictly-more-likely mass is at most top_p are kept; the token is
 //                     read off the cumulative distribution (in index order) at u in [0,1).
 // The uniform number u comes from the host, one per row, so that a request's random
 // stream does not depend on what else is in the batch.
+//
+// Probability masses are summed as 64-bit fixed-point integers (exp(.) * 2^40): integer
+// sums do not depend on the order of addition, so the kept set and the chosen token are
+// the same on every run, however the work is spread over threads, and no rounding can
+// leave the cumulative sum short of its target.
+//
+// argmax alone runs in two launches, many workgroups per row and then a merge.  sample
+// runs one workgroup per row in about five passes over the row:
+//   1. the maximum (and its index);
+//   2. the total mass and, for top_p < 1, a histogram of mass over 2048 bins that are
+//      monotone in the logit, which names the one bin the top-p boundary falls into;
+//   3. the tokens of that bin are gathered in LDS and the exact boundary key is found
+//      there by bisection (if they do not fit, by bisection with passes over the row);
+//   4. the cumulative mass of kept tokens in index order, narrowed from the row to a
+//      sixteenth of it twice and then scanned.
 #include "common.h"
 
+typedef unsigned long long u64;
+
 #define SAMPLE_THREADS 1024
+#define SAMPLE_WAVES (SAMPLE_THREADS / PYLON_WAVE)
+#define ARGMAX_THREADS 256
+#define ARGMAX_MAX_CHUNKS 64
+#define ARGMAX_MIN_CHUNK 1024
+#define BINS 2048
+#define CANDIDATES 4096
+#define FIXED_ONE 1099511627776.0f  // 2^40
+// exp(-28) * 2^40 < 1: a token that far below the maximum has no mass in fixed point.
+#define BIN_RANGE 28.0f
 
 // Order-preserving map from float to unsigned: a < b  <=>  key(a) < key(b).
 __device__ __forceinline__ uint32_t float_key(float f) {
   const uint32_t u = __float_as_uint(f);
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
+
+__device__ __forceinline__ float clean(float x) { return x != x ? -INFINITY : x; }
 
 struct ArgBest {
   float value;
@@ -25,12 +53,39 @@ __device__ __forceinline__ ArgBest better(ArgBest a, ArgBest b) {
   return a;
 }
 
-__device__ int block_argmax(const float* __restrict__ row, int vocab, ArgBest* scratch) {
-  ArgBest best = {-INFINITY, 0x7fffffff};
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-    const float v = row[i];
-    if (v > best.value || best.index == 0x7fffffff) best = {v, i};
+// f(value, index) for every element of row[begin, end), spread over the workgroup's
+// threads in no particular order, with 16-byte loads where the address allows.
+template <typename F>
+__device__ __forceinline__ void for_each(const float* __restrict__ row, int begin, int end, F f) {
+  const float* p = row + begin;
+  const int n = end - begin;
+  int head = static_cast<int>((4 - ((reinterpret_cast<uintptr_t>(p) >> 2) & 3)) & 3);
+  if (head > n) head = n;
+  if (static_cast<int>(threadIdx.x) < head) f(p[threadIdx.x], begin + static_cast<int>(threadIdx.x));
+  const float4* v = reinterpret_cast<const float4*>(p + head);
+  const int nv = (n - head) >> 2;
+#pragma unroll 4
+  for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+    const float4 q = v[i];
+    const int base = begin + head + 4 * i;
+    f(q.x, base);
+    f(q.y, base + 1);
+    f(q.z, base + 2);
+    f(q.w, base + 3);
   }
+  const int tail = head + 4 * nv;
+  if (static_cast<int>(threadIdx.x) < n - tail)
+    f(p[tail + threadIdx.x], begin + tail + static_cast<int>(threadIdx.x));
+}
+
+// The largest element of row[begin, end) and its lowest index, for every thread.
+// NaN counts as -inf; an empty or all -inf range gives index 0x7fffffff or its first index.
+__device__ ArgBest block_argbest(const float* __restrict__ row, int begin, int end, ArgBest* scratch) {
+  ArgBest best = {-INFINITY, 0x7fffffff};
+  for_each(row, begin, end, [&](float v, int i) {
+    v = clean(v);
+    if (v > best.value || (v == best.value && i < best.index)) best = {v, i};
+  });
   for (int off = PYLON_WAVE / 2; off > 0; off >>= 1) {
     ArgBest other;
     other.value = __shfl_xor(best.value, off, PYLON_WAVE);
@@ -44,7 +99,7 @@ __device__ int block_argmax(const float* __restrict__ row, int vocab, ArgBest* s
   ArgBest total = scratch[0];
   const int nwaves = (blockDim.x + PYLON_WAVE - 1) / PYLON_WAVE;
   for (int i = 1; i < nwaves; ++i) total = better(total, scratch[i]);
-  return total.index;
+  return total;
 }
 
 // The chosen id goes to out[row] and, if asked for, also to chosen[place[row]]: a table
@@ -55,129 +110,336 @@ __device__ __forceinline__ void emit(int* __restrict__ out, int* __restrict__ ch
   if (chosen != nullptr) chosen[place[row]] = id;
 }
 
-__global__ __launch_bounds__(SAMPLE_THREADS) void argmax_kernel(int* __restrict__ out,
-                                                                const float* __restrict__ logits,
-                                                                int vocab, long long row_stride,
-                                                                int* __restrict__ chosen,
-                                                                const int* __restrict__ place) {
-  __shared__ ArgBest scratch[16];
-  const float* row = logits + static_cast<size_t>(blockIdx.x) * row_stride;
-  const int idx = block_argmax(row, vocab, scratch);
-  if (threadIdx.x == 0) emit(out, chosen, place, blockIdx.x, idx);
+// ---- argmax: many workgroups per row, then a merge -------------------------------------
+__global__ __launch_bounds__(ARGMAX_THREADS) void argmax_partial_kernel(
+    ArgBest* __restrict__ partial, const float* __restrict__ logits, int vocab, long long row_stride,
+    int chunk_len) {
+  __shared__ ArgBest scratch[ARGMAX_THREADS / PYLON_WAVE];
+  const int r = blockIdx.y, c = blockIdx.x;
+  const float* row = logits + static_cast<size_t>(r) * row_stride;
+  const int begin = c * chunk_len;
+  const int end = begin + chunk_len < vocab ? begin + chunk_len : vocab;
+  const ArgBest best = block_argbest(row, begin, end, scratch);
+  if (threadIdx.x == 0) partial[static_cast<size_t>(r) * gridDim.x + c] = best;
+}
+
+__global__ __launch_bounds__(PYLON_WAVE) void argmax_merge_kernel(
+    int* __restrict__ out, const ArgBest* __restrict__ partial, int chunks, int* __restrict__ chosen,
+    const int* __restrict__ place) {
+  const int r = blockIdx.x;
+  ArgBest best = {-INFINITY, 0x7fffffff};
+  for (int c = threadIdx.x; c < chunks; c += PYLON_WAVE)
+    best = better(best, partial[static_cast<size_t>(r) * chunks + c]);
+  for (int off = PYLON_WAVE / 2; off > 0; off >>= 1) {
+    ArgBest other;
+    other.value = __shfl_xor(best.value, off, PYLON_WAVE);
+    other.index = __shfl_xor(best.index, off, PYLON_WAVE);
+    best = better(best, other);
+  }
+  if (threadIdx.x == 0) emit(out, chosen, place, r, best.index == 0x7fffffff ? 0 : best.index);
+}
+
+extern "C" long long pylon_argmax_scratch_bytes(int rows) {
+  return static_cast<long long>(rows > 0 ? rows : 0) * ARGMAX_MAX_CHUNKS * sizeof(ArgBest);
 }
 
 // chosen and place are both null or both given (place: one index into chosen per row).
+// scratch: device memory of at least pylon_argmax_scratch_bytes(rows) bytes.
 extern "C" int pylon_argmax(int* out, const float* logits, int rows, int vocab, long long row_stride,
-                            int* chosen, const int* place, hipStream_t stream) {
+                            int* chosen, const int* place, void* scratch, long long scratch_bytes,
+                            hipStream_t stream) {
   PYLON_REQUIRE((chosen == nullptr) == (place == nullptr), "argmax: chosen and place go together");
   PYLON_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "argmax: bad sizes rows=%d vocab=%d", rows, vocab);
   if (rows == 0) return 0;
-  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, out, logits, vocab,
-                     row_stride, chosen, place);
+  PYLON_REQUIRE(rows <= 65535, "argmax: at most 65535 rows, got %d", rows);
+  PYLON_REQUIRE(scratch != nullptr && scratch_bytes >= pylon_argmax_scratch_bytes(rows),
+                "argmax: scratch must hold %lld bytes", pylon_argmax_scratch_bytes(rows));
+  int chunks = vocab / ARGMAX_MIN_CHUNK;
+  chunks = chunks < 1 ? 1 : (chunks > ARGMAX_MAX_CHUNKS ? ARGMAX_MAX_CHUNKS : chunks);
+  const int chunk_len = (((vocab + chunks - 1) / chunks) + 3) & ~3;
+  chunks = (vocab + chunk_len - 1) / chunk_len;
+  hipLaunchKernelGGL(argmax_partial_kernel, dim3(chunks, rows), dim3(ARGMAX_THREADS), 0, stream,
+                     static_cast<ArgBest*>(scratch), logits, vocab, row_stride, chunk_len);
+  hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(PYLON_WAVE), 0, stream, out,
+                     static_cast<const ArgBest*>(scratch), chunks, chosen, place);
   PYLON_LAUNCHED("argmax");
+}
+
+// ---- sample ------------------------------------------------------------------------------
+__device__ __forceinline__ u64 wave_sum_u64(u64 v) {
+#pragma unroll
+  for (int off = PYLON_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, PYLON_WAVE);
+  return v;
+}
+
+// Sum over the workgroup, for every thread.  `scratch` holds SAMPLE_WAVES values.
+__device__ __forceinline__ u64 block_sum_u64(u64 v, u64* scratch) {
+  const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
+  v = wave_sum_u64(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  u64 total = 0;
+  for (int i = 0; i < SAMPLE_WAVES; ++i) total += scratch[i];
+  return total;
+}
+
+// A token's probability mass relative to the most likely one, in units of 2^-40.
+__device__ __forceinline__ u64 mass_of(float x, float mx, float inv_temp) {
+  return static_cast<u64>(expf((x - mx) * inv_temp) * FIXED_ONE);
+}
+
+// Bin 0 holds the most likely tokens; a larger logit never lands in a later bin.
+__device__ __forceinline__ int bin_of(float x, float mx, float inv_temp) {
+  const float t = (mx - x) * inv_temp * (BINS / BIN_RANGE);
+  return t >= static_cast<float>(BINS - 1) ? BINS - 1 : static_cast<int>(t);
+}
+
+// Four consecutive logits from index i (a multiple of 4 past an aligned row), -inf past `end`.
+__device__ __forceinline__ float4 load_four(const float* __restrict__ row, int i, int end, bool aligned) {
+  if (aligned && i + 3 < end) return *reinterpret_cast<const float4*>(row + i);
+  float4 v;
+  v.x = i < end ? row[i] : -INFINITY;
+  v.y = i + 1 < end ? row[i + 1] : -INFINITY;
+  v.z = i + 2 < end ? row[i + 2] : -INFINITY;
+  v.w = i + 3 < end ? row[i + 3] : -INFINITY;
+  return v;
 }
 
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     int* __restrict__ out, const float* __restrict__ logits, int vocab, long long row_stride,
     const float* __restrict__ temperature, const float* __restrict__ top_p,
     const float* __restrict__ uniform, int* __restrict__ chosen, const int* __restrict__ place) {
-  __shared__ ArgBest best_scratch[16];
-  __shared__ float scratch[16];
-  __shared__ float wave_totals[16];
-  __shared__ int found;
+  // The histogram first; once the boundary bin is known, that bin's tokens (key, mass).
+  __shared__ __align__(16) unsigned char pool[CANDIDATES * (sizeof(uint32_t) + sizeof(u64))];
+  __shared__ ArgBest best_scratch[SAMPLE_WAVES];
+  __shared__ u64 sum_scratch[SAMPLE_WAVES];
+  __shared__ u64 seg_total[SAMPLE_WAVES];
+  __shared__ u64 shared_mass[2];  // [0]: mass in the bins before the boundary bin; [1]: kept mass
+  __shared__ int shared_bin;
+  __shared__ int cand_count;
+  __shared__ uint32_t key_range[2];
+  __shared__ uint32_t shared_threshold;
+
   const int r = blockIdx.x;
   const float* row = logits + static_cast<size_t>(r) * row_stride;
+  const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
   const float temp = temperature[r];
-  if (temp <= 0.f) {
-    const int idx = block_argmax(row, vocab, best_scratch);
-    if (threadIdx.x == 0) emit(out, chosen, place, r, idx);
+
+  // pass 1
+  const ArgBest top = block_argbest(row, 0, vocab, best_scratch);
+  const int top_index = top.index == 0x7fffffff ? 0 : top.index;
+  const float mx = top.value;
+  if (temp <= 0.f || !(mx > -INFINITY) || !(mx < INFINITY)) {
+    if (threadIdx.x == 0) emit(out, chosen, place, r, top_index);
     return;
   }
   const float inv_temp = 1.0f / temp;
-  float mx = -INFINITY;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) mx = fmaxf(mx, row[i]);
-  mx = block_max(mx, scratch);
-  float z = 0.f;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) z += expf((row[i] - mx) * inv_temp);
-  z = block_sum(z, scratch);
+  const float p = top_p[r];
+  const bool restricted = p < 1.0f;
+
+  // pass 2
+  u64* hist = reinterpret_cast<u64*>(pool);
+  if (restricted) {
+    for (int b = threadIdx.x; b < BINS; b += SAMPLE_THREADS) hist[b] = 0;
+    if (threadIdx.x == 0) {
+      cand_count = 0;
+      key_range[0] = 0xffffffffu;
+      key_range[1] = 0;
+    }
+    __syncthreads();
+  }
+  u64 zq = 0;
+  for_each(row, 0, vocab, [&](float x, int) {
+    x = clean(x);
+    const u64 q = mass_of(x, mx, inv_temp);
+    zq += q;
+    if (restricted && q != 0) atomicAdd(&hist[bin_of(x, mx, inv_temp)], q);
+  });
+  zq = block_sum_u64(zq, sum_scratch);  // >= 2^40: the maximum itself
 
   uint32_t threshold = 0;  // tokens with key >= threshold are kept
-  float kept_mass = z;
-  const float p = top_p[r];
-  if (p < 1.0f) {
-    const float target = p * z;
-    uint32_t lo = 0, hi = float_key(mx);
-    while (lo < hi) {
-      const uint32_t mid = lo + (hi - lo) / 2;
-      float above = 0.f;
-      for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-        const float v = row[i];
-        if (float_key(v) > mid) above += expf((v - mx) * inv_temp);
+  u64 kept_mass = zq;
+  if (restricted) {
+    u64 target = static_cast<u64>(static_cast<double>(p) * static_cast<double>(zq));
+    if (target >= zq) target = zq - 1;
+    // The boundary bin: mass before it <= target < mass before it + its own mass.
+    if (wave == 0) {
+      constexpr int PER_LANE = BINS / PYLON_WAVE;
+      u64 mine = 0;
+      for (int j = 0; j < PER_LANE; ++j) mine += hist[lane * PER_LANE + j];
+      u64 scan = mine;
+      for (int off = 1; off < PYLON_WAVE; off <<= 1) {
+        const u64 up = __shfl_up(scan, off, PYLON_WAVE);
+        if (lane >= off) scan += up;
       }
-      above = block_sum(above, scratch);
-      if (above <= target)
-        hi = mid;
-      else
-        lo = mid + 1;
+      u64 before = scan - mine;
+      for (int j = 0; j < PER_LANE; ++j) {
+        const u64 h = hist[lane * PER_LANE + j];
+        if (before <= target && target < before + h) {
+          shared_bin = lane * PER_LANE + j;
+          shared_mass[0] = before;
+        }
+        before += h;
+      }
     }
-    threshold = lo;
-    float kept = 0.f;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-      const float v = row[i];
-      if (float_key(v) >= threshold) kept += expf((v - mx) * inv_temp);
+    __syncthreads();
+    const int boundary = shared_bin;
+    const u64 before_bin = shared_mass[0];
+    __syncthreads();  // the histogram is read; its memory now takes the bin's tokens
+
+    // pass 3
+    uint32_t* cand_key = reinterpret_cast<uint32_t*>(pool);
+    u64* cand_mass = reinterpret_cast<u64*>(pool + CANDIDATES * sizeof(uint32_t));
+    for_each(row, 0, vocab, [&](float x, int) {
+      x = clean(x);
+      if (bin_of(x, mx, inv_temp) != boundary) return;
+      const u64 q = mass_of(x, mx, inv_temp);
+      if (q == 0) return;
+      const uint32_t key = float_key(x);
+      atomicMin(&key_range[0], key);
+      atomicMax(&key_range[1], key);
+      const int at = atomicAdd(&cand_count, 1);
+      if (at < CANDIDATES) {
+        cand_key[at] = key;
+        cand_mass[at] = q;
+      }
+    });
+    __syncthreads();
+    const int count = cand_count;
+    // The smallest key k with (mass of keys > k) <= target lies in [lo, hi]: at hi only the
+    // earlier bins are above, at lo - 1 the whole boundary bin would be as well.
+    uint32_t lo = key_range[0], hi = key_range[1];
+    if (count <= CANDIDATES) {
+      if (wave == 0) {
+        while (lo < hi) {
+          const uint32_t mid = lo + (hi - lo) / 2;
+          u64 above = 0;
+          for (int j = lane; j < count; j += PYLON_WAVE)
+            if (cand_key[j] > mid) above += cand_mass[j];
+          above = before_bin + wave_sum_u64(above);
+          if (above <= target)
+            hi = mid;
+          else
+            lo = mid + 1;
+        }
+        u64 kept = 0;
+        for (int j = lane; j < count; j += PYLON_WAVE)
+          if (cand_key[j] >= lo) kept += cand_mass[j];
+        kept = before_bin + wave_sum_u64(kept);
+        if (lane == 0) {
+          shared_threshold = lo;
+          shared_mass[1] = kept;
+        }
+      }
+      __syncthreads();
+      threshold = shared_threshold;
+      kept_mass = shared_mass[1];
+    } else {
+      // More tokens in one bin than LDS holds (thousands of near-equal logits): bisect
+      // with a pass over the row for each probe.
+      while (lo < hi) {
+        const uint32_t mid = lo + (hi - lo) / 2;
+        u64 above = 0;
+        for_each(row, 0, vocab, [&](float x, int) {
+          x = clean(x);
+          if (float_key(x) > mid) above += mass_of(x, mx, inv_temp);
+        });
+        above = block_sum_u64(above, sum_scratch);
+        if (above <= target)
+          hi = mid;
+        else
+          lo = mid + 1;
+      }
+      threshold = lo;
+      u64 kept = 0;
+      for_each(row, 0, vocab, [&](float x, int) {
+        x = clean(x);
+        if (float_key(x) >= threshold) kept += mass_of(x, mx, inv_temp);
+      });
+      kept_mass = block_sum_u64(kept, sum_scratch);
     }
-    kept_mass = block_sum(kept, scratch);
   }
 
-  const float target = uniform[r] * kept_mass;
-  if (threadIdx.x == 0) found = 0x7fffffff;
-  __syncthreads();
-  const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
-  const int nwaves = blockDim.x / PYLON_WAVE;
-  float running = 0.f;
-  int last_kept = -1;
-  for (int base = 0; base < vocab; base += blockDim.x) {
-    const int i = base + threadIdx.x;
-    float e = 0.f;
-    if (i < vocab) {
-      const float v = row[i];
-      if (float_key(v) >= threshold) {
-        e = expf((v - mx) * inv_temp);
-        last_kept = i;
+  // pass 4: the first index, in index order, at which the cumulative kept mass exceeds
+  // u * (kept mass).
+  float u = uniform[r];
+  u = u < 0.f ? 0.f : u;
+  u64 target = static_cast<u64>(static_cast<double>(u) * static_cast<double>(kept_mass));
+  if (target >= kept_mass) target = kept_mass - 1;
+  const bool aligned = (reinterpret_cast<uintptr_t>(row) & 15) == 0;
+  auto kept_mass_of = [&](float x) -> u64 {
+    x = clean(x);
+    return float_key(x) >= threshold ? mass_of(x, mx, inv_temp) : 0;
+  };
+  int begin = 0, end = vocab;
+  u64 before = 0;
+  bool lost = false;
+  while (end - begin > 4 * PYLON_WAVE * 4) {
+    // sixteen consecutive stretches, one per wave
+    int seg = (end - begin + SAMPLE_WAVES - 1) / SAMPLE_WAVES;
+    seg = (seg + 4 * PYLON_WAVE - 1) / (4 * PYLON_WAVE) * (4 * PYLON_WAVE);
+    const int s0 = begin + wave * seg;
+    const int s1 = s0 + seg < end ? s0 + seg : end;
+    u64 mine = 0;
+#pragma unroll 4
+    for (int i = s0 + 4 * lane; i < s1; i += 4 * PYLON_WAVE) {
+      const float4 v = load_four(row, i, s1, aligned);
+      mine += kept_mass_of(v.x) + kept_mass_of(v.y) + kept_mass_of(v.z) + kept_mass_of(v.w);
+    }
+    mine = wave_sum_u64(mine);
+    __syncthreads();
+    if (lane == 0) seg_total[wave] = mine;
+    __syncthreads();
+    int pick = -1;
+    for (int w = 0; w < SAMPLE_WAVES; ++w) {
+      const u64 t = seg_total[w];
+      if (before + t > target) {
+        pick = w;
+        break;
+      }
+      before += t;
+    }
+    if (pick < 0) {
+      lost = true;
+      break;
+    }
+    begin += pick * seg;
+    end = begin + seg < end ? begin + seg : end;
+  }
+  if (lost) {  // cannot happen while the masses are summed as integers; never leave out[] unset
+    if (threadIdx.x == 0) emit(out, chosen, place, r, top_index);
+    return;
+  }
+  if (wave == 0) {
+    int found = -1;
+    for (int sub = begin; sub < end && found < 0; sub += 4 * PYLON_WAVE) {
+      const int i = sub + 4 * lane;
+      const float4 v = load_four(row, i, end, aligned);
+      const u64 q0 = kept_mass_of(v.x), q1 = kept_mass_of(v.y), q2 = kept_mass_of(v.z), q3 = kept_mass_of(v.w);
+      const u64 mine = q0 + q1 + q2 + q3;
+      u64 scan = mine;
+      for (int off = 1; off < PYLON_WAVE; off <<= 1) {
+        const u64 up = __shfl_up(scan, off, PYLON_WAVE);
+        if (lane >= off) scan += up;
+      }
+      const u64 crossing = __ballot(before + scan > target);
+      if (crossing != 0) {
+        const int first = __ffsll(static_cast<long long>(crossing)) - 1;
+        int index = -1;
+        if (lane == first) {
+          u64 cum = before + scan - mine;
+          if (cum + q0 > target) index = i;
+          else if (cum + q0 + q1 > target) index = i + 1;
+          else if (cum + q0 + q1 + q2 > target) index = i + 2;
+          else index = i + 3;
+        }
+        found = __shfl(index, first, PYLON_WAVE);
+      } else {
+        before += __shfl(scan, PYLON_WAVE - 1, PYLON_WAVE);
       }
     }
-    // inclusive scan over the workgroup
-    float scan = e;
-    for (int off = 1; off < PYLON_WAVE; off <<= 1) {
-      const float up = __shfl_up(scan, off, PYLON_WAVE);
-      if (lane >= off) scan += up;
-    }
-    if (lane == PYLON_WAVE - 1) wave_totals[wave] = scan;
-    __syncthreads();
-    float before = running;
-    for (int wv = 0; wv < wave; ++wv) before += wave_totals[wv];
-    float tile_total = 0.f;
-    for (int wv = 0; wv < nwaves; ++wv) tile_total += wave_totals[wv];
-    const float cum = before + scan;
-    if (e > 0.f && cum > target) atomicMin(&found, i);
-    __syncthreads();
-    if (found != 0x7fffffff) break;
-    running += tile_total;
-  }
-  if (found == 0x7fffffff) {
-    // Rounding left the cumulative sum just below the target: take the last kept token.
-    int lk = last_kept;
-    for (int off = PYLON_WAVE / 2; off > 0; off >>= 1) lk = max(lk, __shfl_xor(lk, off, PYLON_WAVE));
-    __shared__ int last_scratch[16];
-    if (lane == 0) last_scratch[wave] = lk;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      int v = -1;
-      for (int wv = 0; wv < nwaves; ++wv) v = max(v, last_scratch[wv]);
-      emit(out, chosen, place, r, v < 0 ? 0 : v);
-    }
-  } else if (threadIdx.x == 0) {
-    emit(out, chosen, place, r, found);
+    if (lane == 0) emit(out, chosen, place, r, found < 0 ? top_index : found);
   }
 }
 

@@ -438,8 +438,10 @@ def argmax(logits: torch.Tensor, *, out: Optional[torch.Tensor] = None,
         raise KernelError("argmax takes float32 logits on the GPU")
     out = _ids_out(rows, logits.device, out)
     chosen_ptr, place_ptr = _chosen_args(rows, chosen, place)
+    # the first launch leaves up to 64 partial results of 8 bytes per row for the second
+    scratch = torch.empty((max(rows, 1) * 64 * 8,), dtype=torch.uint8, device=logits.device)
     _lib.call("pylon_argmax", out.data_ptr(), logits.data_ptr(), rows, vocab, logits.stride(0),
-              chosen_ptr, place_ptr, _stream())
+              chosen_ptr, place_ptr, scratch.data_ptr(), scratch.numel(), _stream())
     return out
 
 

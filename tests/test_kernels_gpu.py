@@ -523,6 +523,90 @@ def test_sampling_kernels(ops):
     assert np.abs(freq - [0.5, 0.25, 0.125, 0.125]).max() < 0.03
 
 
+def _check_draws(ops, logits, temps, tops, us, plain):
+    """Every draw is the plain rule's, or an adjacent kept token with u on that boundary of
+    the cumulative distribution."""
+    got = ops.sample(logits.to(DEV), temps.to(DEV), tops.to(DEV), us.to(DEV)).cpu().tolist()
+    again = ops.sample(logits.to(DEV), temps.to(DEV), tops.to(DEV), us.to(DEV)).cpu().tolist()
+    assert got == again  # integer masses: the same on every run
+    for r in range(logits.shape[0]):
+        row = f64(logits)[r]
+        want = plain.sample_with_uniform(row, float(temps[r]), float(tops[r]), float(us[r]))
+        if got[r] != want:
+            p = plain.sampling_distribution(row, float(temps[r]), float(tops[r]))
+            cdf = np.cumsum(p)
+            assert p[got[r]] > 0 and abs(cdf[min(got[r], want)] - float(us[r])) < 1e-5, (r, got[r], want)
+    return got
+
+
+def test_sampling_at_a_full_vocabulary_and_odd_layouts(ops):
+    from tests.plain import qwen3 as plain
+
+    # a real vocabulary; rows that start at addresses that are no multiple of 16 bytes
+    vocab = 151936
+    base = rnd((5, vocab + 3), 41, scale=2.5)
+    logits = base[:, 1: 1 + vocab]  # row stride vocab + 3, first element off by one float
+    assert logits.stride(0) == vocab + 3
+    dev_base = base.to(DEV)
+    dev = dev_base[:, 1: 1 + vocab]
+    temps = torch.tensor([1.0, 0.6, 0.2, 1.5, 0.9])
+    tops = torch.tensor([0.95, 0.5, 0.95, 1.0, 0.999])
+    assert ops.argmax(dev).cpu().tolist() == f64(logits).argmax(axis=1).tolist()
+    for trial in range(4):
+        us = torch.rand(5, generator=torch.Generator().manual_seed(7 + trial))
+        got = ops.sample(dev, temps.to(DEV), tops.to(DEV), us.to(DEV)).cpu().tolist()
+        for r in range(5):
+            row = f64(logits)[r]
+            want = plain.sample_with_uniform(row, float(temps[r]), float(tops[r]), float(us[r]))
+            if got[r] != want:
+                p = plain.sampling_distribution(row, float(temps[r]), float(tops[r]))
+                cdf = np.cumsum(p)
+                assert p[got[r]] > 0 and abs(cdf[min(got[r], want)] - float(us[r])) < 1e-5, (trial, r)
+    # the kept set: u just below 1 draws the last kept token in vocabulary order
+    almost_one = torch.full((5,), 1.0 - 2 ** -24)
+    got = ops.sample(dev, temps.to(DEV), tops.to(DEV), almost_one.to(DEV)).cpu().tolist()
+    for r in range(5):
+        p = plain.sampling_distribution(f64(logits)[r], float(temps[r]), float(tops[r]))
+        kept = np.nonzero(p > 2.0 ** -40)[0]
+        assert got[r] == int(kept[-1]), r
+    # u = 0 draws the first kept token
+    got = ops.sample(dev, temps.to(DEV), tops.to(DEV), torch.zeros(5, device=DEV)).cpu().tolist()
+    for r in range(5):
+        p = plain.sampling_distribution(f64(logits)[r], float(temps[r]), float(tops[r]))
+        assert got[r] == int(np.nonzero(p > 2.0 ** -40)[0][0]), r
+
+
+def test_sampling_with_thousands_of_equal_logits_at_the_boundary(ops):
+    """More tokens in the top-p boundary's bin than the kernel gathers in LDS, most of them
+    equal: the kept set is still the rule's (a tie is kept or dropped as a whole)."""
+    from tests.plain import qwen3 as plain
+
+    vocab = 20000
+    gen = torch.Generator().manual_seed(5)
+    logits = torch.full((3, vocab), -4.0)
+    logits[:, :50] = 2.0 + torch.rand((3, 50), generator=gen)  # a head that holds ~60 % of the mass
+    logits[:, 50:9000] = 0.0                                       # 8950 equal tokens
+    logits[1, 50:9000] += torch.rand(8950, generator=gen) * 1e-3   # ... or nearly equal
+    logits[2, 9000:] = -30.0
+    temps = torch.ones(3)
+    for top_p in (0.7, 0.95):
+        tops = torch.full((3,), top_p)
+        dev = logits.to(DEV)
+        almost_one = torch.full((3,), 1.0 - 2 ** -24)
+        last = ops.sample(dev, temps.to(DEV), tops.to(DEV), almost_one.to(DEV)).cpu().tolist()
+        first = ops.sample(dev, temps.to(DEV), tops.to(DEV), torch.zeros(3, device=DEV)).cpu().tolist()
+        for r in range(3):
+            row = f64(logits)[r]
+            p = np.exp(row - row.max())
+            p /= p.sum()
+            above = np.array([p[row > x].sum() for x in np.unique(row)])
+            keep_values = np.unique(row)[above <= top_p + 1e-12]
+            kept = np.nonzero(np.isin(row, keep_values) & (p * 2.0 ** 40 / p.max() >= 1))[0]
+            assert first[r] == int(kept[0]) and last[r] == int(kept[-1]), (top_p, r, first[r], last[r])
+    us = torch.tensor([0.3, 0.6, 0.9])
+    _check_draws(ops, logits[1:2].repeat(3, 1), temps, torch.full((3,), 0.7), us, plain)
+
+
 def test_kernels_refuse_what_they_cannot_do(ops):
     from pylon_amd.kernels import KernelError
 
