@@ -14,7 +14,14 @@
 // runs on the vector units: a value row is read by head_dim/8 lanes, 16 bytes each, so one
 // load instruction fetches the rows of several keys; every lane accumulates its eight
 // elements over its keys and the lane groups are summed at the end.  Softmax statistics are float throughout.
+//
+// The kernel can also take over the step that precedes attention: given the raw q/k/v
+// projection instead of prepared queries, each workgroup first norms and rotates its
+// group's query heads (kept in LDS) and its key head, stores that key and its value head
+// at the token's cache slot, and only then reads the cache, the new key included.  One
+// launch and one pass over the projection less per layer.
 #include "common.h"
+#include "head_prepare.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -24,13 +31,42 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 #define AD_SUPER 64  // keys whose loads are in flight together (four score tiles)
 #define AD_MAX_WAVES 8
 
+// What the kernel needs to prepare q, k and v itself (PREP): the raw projection
+// [tokens, row_stride] with q heads first, then k heads, then v heads.
+struct DecodePrep {
+  const uint16_t* qkv;
+  long long row_stride;
+  const float* q_weight;  // per-head RMSNorm weights, or null
+  const float* k_weight;
+  float eps;
+  const float* inv_freq;  // head_dim/2 rotation frequencies, or null
+  const int* slot_map;    // cache slot of each token's key and value; null: store nothing
+};
+
+// With PREP the kernel writes the caches before it reads them, so they are neither const
+// nor restrict there.
+template <bool PREP>
+struct DecodeCache {
+  typedef const uint16_t* __restrict__ ptr;
+};
+template <>
+struct DecodeCache<true> {
+  typedef uint16_t* ptr;
+};
+
+static __host__ __device__ size_t decode_lds_floats(int n_waves, int gp, int head_dim) {
+  const size_t n = static_cast<size_t>(n_waves) * AD_SUPER * gp + static_cast<size_t>(n_waves) * gp * head_dim +
+                   static_cast<size_t>(n_waves) * gp * 2;
+  return (n + 3) & ~static_cast<size_t>(3);  // what follows stays 16-byte aligned
+}
+
 // EPL = head_dim / 64, KSTEPS = head_dim / 32, GP = heads per group rounded up to 1, 2, 4, 8, 16
-template <int EPL, int KSTEPS, int GP>
+template <int EPL, int KSTEPS, int GP, bool PREP>
 __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_kernel(
-    uint16_t* __restrict__ out, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
-    const uint16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
+    uint16_t* __restrict__ out, const uint16_t* __restrict__ q, typename DecodeCache<PREP>::ptr k_cache,
+    typename DecodeCache<PREP>::ptr v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tok_row, const int* __restrict__ positions, int n_heads, int n_kv_heads,
-    int page_size, int window, float scale) {
+    int page_size, int window, float scale, DecodePrep prep) {
   constexpr int HD = EPL * 64;
   constexpr int TILES = AD_SUPER / AD_TILE;
   // per wave: probabilities of the keys in flight; then the waves' partial results
@@ -41,6 +77,7 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
   float(*p_tile)[GP] = reinterpret_cast<float(*)[GP]>(lds + wave * AD_SUPER * GP);
   float* part_acc = lds + n_waves * AD_SUPER * GP;  // [wave][GP][HD]
   float* part_ml = part_acc + n_waves * GP * HD;    // [wave][GP][2]
+  uint16_t* q_lds = reinterpret_cast<uint16_t*>(lds + decode_lds_floats(n_waves, GP, HD));  // [GP][HD], PREP only
   const int col = lane & 15, grp = lane >> 4;
   const int kvh = blockIdx.x, t = blockIdx.y;
   const int group = n_heads / n_kv_heads;
@@ -60,11 +97,37 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
   int k_end = k_begin + per_wave;
   if (k_end > pos + 1) k_end = pos + 1;
 
+  if constexpr (PREP) {
+    // One wave per head: the group's query heads into LDS, then this key head and this
+    // value head into the token's cache slot.
+    const uint16_t* row = prep.qkv + static_cast<size_t>(t) * prep.row_stride;
+    const int slot = prep.slot_map != nullptr ? prep.slot_map[t] : -1;
+    const int jobs = group + (slot >= 0 ? 2 : 0);
+    const float fpos = static_cast<float>(pos);
+    for (int job = wave; job < jobs; job += n_waves) {
+      float v[EPL];
+      if (job < group) {
+        load_head_bf16<EPL>(row + static_cast<size_t>(kvh * group + job) * HD, lane, v);
+        norm_rotate_head<EPL>(v, lane, prep.q_weight, prep.eps, prep.inv_freq, fpos);
+        store_head_bf16<EPL>(q_lds + job * HD, lane, v);
+      } else {
+        const bool is_key = job == group;
+        load_head_bf16<EPL>(row + static_cast<size_t>(n_heads + (is_key ? 0 : n_kv_heads) + kvh) * HD, lane, v);
+        if (is_key) norm_rotate_head<EPL>(v, lane, prep.k_weight, prep.eps, prep.inv_freq, fpos);
+        uint16_t* dst = (is_key ? k_cache : v_cache) + (static_cast<size_t>(slot) * n_kv_heads + kvh) * HD;
+        store_head_bf16<EPL>(dst, lane, v);
+      }
+    }
+    // The barrier orders the workgroup's stores before its loads: every wave sees the new
+    // key and value in the cache and the queries in LDS.
+    __syncthreads();
+  }
   // query fragments: column `col` is head kvh*group + col of the token
   bf16x8 qf[KSTEPS];
   {
     const bool valid = col < group;
-    const uint16_t* qrow = q + (static_cast<size_t>(t) * n_heads + kvh * group + (valid ? col : 0)) * HD;
+    const uint16_t* qrow = PREP ? q_lds + (valid ? col : 0) * HD
+                                : q + (static_cast<size_t>(t) * n_heads + kvh * group + (valid ? col : 0)) * HD;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       if (valid) {
@@ -220,26 +283,27 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
   }
 }
 
-static size_t decode_lds_bytes(int n_waves, int gp, int head_dim) {
-  return sizeof(float) * (static_cast<size_t>(n_waves) * AD_SUPER * gp +
-                          static_cast<size_t>(n_waves) * gp * head_dim + static_cast<size_t>(n_waves) * gp * 2);
+static size_t decode_lds_bytes(int n_waves, int gp, int head_dim, bool prep) {
+  return sizeof(float) * decode_lds_floats(n_waves, gp, head_dim) +
+         (prep ? sizeof(uint16_t) * static_cast<size_t>(gp) * head_dim : 0);
 }
 
-template <int EPL>
-static int launch_decode(void* out, const void* q, const void* k_cache, const void* v_cache,
+template <int EPL, bool PREP>
+static int launch_decode(void* out, const void* q, void* k_cache, void* v_cache,
                          const int* block_table, int table_width, const int* tok_row,
                          const int* positions, int tokens, int n_heads, int n_kv_heads, int page_size,
-                         int window, float scale, int n_waves, hipStream_t stream) {
+                         int window, float scale, int n_waves, DecodePrep prep, hipStream_t stream) {
   const int group = n_heads / n_kv_heads;
   const int gp = group <= 1 ? 1 : group <= 2 ? 2 : group <= 4 ? 4 : group <= 8 ? 8 : 16;
   // the partial results of all waves have to fit into 64 KB of LDS
-  while (n_waves > 1 && decode_lds_bytes(n_waves, gp, EPL * 64) > 65536) n_waves /= 2;
-  const size_t lds = decode_lds_bytes(n_waves, gp, EPL * 64);
+  while (n_waves > 1 && decode_lds_bytes(n_waves, gp, EPL * 64, PREP) > 65536) n_waves /= 2;
+  const size_t lds = decode_lds_bytes(n_waves, gp, EPL * 64, PREP);
   dim3 grid(n_kv_heads, tokens), block(n_waves * PYLON_WAVE);
-#define LAUNCH(GP)                                                                                          \
-  hipLaunchKernelGGL((attention_decode_kernel<EPL, EPL * 2, GP>), grid, block, lds, stream, (uint16_t*)out, \
-                     (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_table,   \
-                     table_width, tok_row, positions, n_heads, n_kv_heads, page_size, window, scale)
+#define LAUNCH(GP)                                                                                         \
+  hipLaunchKernelGGL((attention_decode_kernel<EPL, EPL * 2, GP, PREP>), grid, block, lds, stream,          \
+                     (uint16_t*)out, (const uint16_t*)q, (typename DecodeCache<PREP>::ptr)k_cache,         \
+                     (typename DecodeCache<PREP>::ptr)v_cache, block_table, table_width, tok_row, positions, \
+                     n_heads, n_kv_heads, page_size, window, scale, prep)
   switch (gp) {
     case 1: LAUNCH(1); break;
     case 2: LAUNCH(2); break;
@@ -251,6 +315,21 @@ static int launch_decode(void* out, const void* q, const void* k_cache, const vo
   return 0;
 }
 
+static int check_decode_geometry(const char* name, int tokens, int n_heads, int n_kv_heads, int head_dim,
+                                 int page_size, int table_width, int window, int n_waves) {
+  PYLON_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
+                "%s: %d query heads cannot be grouped over %d key/value heads", name, n_heads, n_kv_heads);
+  PYLON_REQUIRE(n_heads / n_kv_heads <= AD_MAX_GROUP, "%s: at most %d query heads per key/value head", name,
+                AD_MAX_GROUP);
+  PYLON_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256, "%s: head_dim %d is not 64, 128 or 256",
+                name, head_dim);
+  PYLON_REQUIRE(page_size > 0 && table_width > 0 && window >= 0, "%s: bad page size, width or window", name);
+  PYLON_REQUIRE(n_waves == 1 || n_waves == 2 || n_waves == 4 || n_waves == 8,
+                "%s: 1, 2, 4 or 8 waves per (token, head), got %d", name, n_waves);
+  PYLON_REQUIRE(tokens <= 65535 && n_kv_heads <= 65535, "%s: too many tokens or heads for one launch", name);
+  return 0;
+}
+
 // q, out: [tokens, n_heads, head_dim] bf16; n_waves (1, 2, 4 or 8) wavefronts share
 // the keys of one (token, key/value head).
 extern "C" int pylon_attention_decode(void* out, const void* q, const void* k_cache, const void* v_cache,
@@ -258,21 +337,15 @@ extern "C" int pylon_attention_decode(void* out, const void* q, const void* k_ca
                                       const int* positions, int tokens, int n_heads, int n_kv_heads,
                                       int head_dim, int page_size, int window, float scale, int n_waves,
                                       hipStream_t stream) {
-  PYLON_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
-                "attention_decode: %d query heads cannot be grouped over %d key/value heads", n_heads,
-                n_kv_heads);
-  PYLON_REQUIRE(n_heads / n_kv_heads <= AD_MAX_GROUP,
-                "attention_decode: at most %d query heads per key/value head", AD_MAX_GROUP);
-  PYLON_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256,
-                "attention_decode: head_dim %d is not 64, 128 or 256", head_dim);
-  PYLON_REQUIRE(page_size > 0 && table_width > 0 && window >= 0, "attention_decode: bad page size, width or window");
-  PYLON_REQUIRE(n_waves == 1 || n_waves == 2 || n_waves == 4 || n_waves == 8,
-                "attention_decode: 1, 2, 4 or 8 waves per (token, head), got %d", n_waves);
-  PYLON_REQUIRE(tokens <= 65535 && n_kv_heads <= 65535, "attention_decode: too many tokens or heads for one launch");
+  if (check_decode_geometry("attention_decode", tokens, n_heads, n_kv_heads, head_dim, page_size, table_width,
+                            window, n_waves))
+    return 1;
   if (tokens == 0) return 0;
-#define GO(D)                                                                                      \
-  launch_decode<D>(out, q, k_cache, v_cache, block_table, table_width, tok_row, positions, tokens, \
-                   n_heads, n_kv_heads, page_size, window, scale, n_waves, stream)
+  const DecodePrep none = {};
+#define GO(D)                                                                                       \
+  launch_decode<D, false>(out, q, const_cast<void*>(k_cache), const_cast<void*>(v_cache), block_table, \
+                          table_width, tok_row, positions, tokens, n_heads, n_kv_heads, page_size, window, \
+                          scale, n_waves, none, stream)
   switch (head_dim / 64) {
     case 1: GO(1); break;
     case 2: GO(2); break;
@@ -280,4 +353,38 @@ extern "C" int pylon_attention_decode(void* out, const void* q, const void* k_ca
   }
 #undef GO
   PYLON_LAUNCHED("attention_decode");
+}
+
+// The same from the raw projection qkv: [tokens, row_stride] bf16 with q heads first, then
+// (if slot_map is given) k heads, then v heads.  Each token's key and value are normed,
+// rotated (inv_freq: head_dim/2 frequencies for a rotation of the whole head, or null) and
+// stored at slot_map[t] before the cache is read; a negative slot stores nothing.  With
+// slot_map null only the queries are prepared (a layer that reads another layer's cache).
+extern "C" int pylon_attention_decode_fused(void* out, const void* qkv, long long row_stride,
+                                            const float* q_weight, const float* k_weight, float eps,
+                                            const float* inv_freq, void* k_cache, void* v_cache,
+                                            const int* slot_map, const int* block_table, int table_width,
+                                            const int* tok_row, const int* positions, int tokens,
+                                            int n_heads, int n_kv_heads, int head_dim, int page_size,
+                                            int window, float scale, int n_waves, hipStream_t stream) {
+  if (check_decode_geometry("attention_decode_fused", tokens, n_heads, n_kv_heads, head_dim, page_size,
+                            table_width, window, n_waves))
+    return 1;
+  const long long heads = n_heads + (slot_map != nullptr ? 2ll * n_kv_heads : 0);
+  PYLON_REQUIRE(row_stride >= heads * head_dim, "attention_decode_fused: row stride %lld is shorter than %lld heads of %d",
+                row_stride, heads, head_dim);
+  PYLON_REQUIRE(row_stride % 2 == 0 && (reinterpret_cast<uintptr_t>(qkv) & 3) == 0,
+                "attention_decode_fused: the projection's rows must be 4-byte aligned");
+  if (tokens == 0) return 0;
+  const DecodePrep prep = {static_cast<const uint16_t*>(qkv), row_stride, q_weight, k_weight, eps, inv_freq, slot_map};
+#define GO(D)                                                                                            \
+  launch_decode<D, true>(out, nullptr, k_cache, v_cache, block_table, table_width, tok_row, positions, tokens, \
+                         n_heads, n_kv_heads, page_size, window, scale, n_waves, prep, stream)
+  switch (head_dim / 64) {
+    case 1: GO(1); break;
+    case 2: GO(2); break;
+    default: GO(4); break;
+  }
+#undef GO
+  PYLON_LAUNCHED("attention_decode_fused");
 }

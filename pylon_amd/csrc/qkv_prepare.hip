@@ -4,6 +4,7 @@
 // pages.  One wavefront handles one head of one token.  Norm, angles and rotation are
 // computed in float and rounded once on the store.
 #include "common.h"
+#include "head_prepare.h"
 
 #define QKV_WAVES 4
 
@@ -140,26 +141,8 @@ __global__ void qkv_prepare_wide_kernel(T* __restrict__ q_out, T* __restrict__ k
 #pragma unroll
     for (int e = 0; e < EPL; ++e) v[e] = to_float(src[lane * EPL + e]);
   }
-  if (weight != nullptr) {
-    float ss = 0.f;
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) ss += v[e] * v[e];
-    ss = wave_sum(ss);
-    const float inv = 1.0f / sqrtf(ss / static_cast<float>(HD) + eps);
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) v[e] = (v[e] * inv) * weight[lane * EPL + e];
-  }
-  if (rotate) {
-    const float pos = static_cast<float>(positions[t]);
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) {
-      const float other = __shfl_xor(v[e], 32, PYLON_WAVE);
-      const int pair = (lane & 31) * EPL + e;  // index of the (i, i + HD/2) pair
-      const float angle = pos * inv_freq[pair];
-      const float c = cosf(angle), sn = sinf(angle);
-      v[e] = (lane < 32) ? v[e] * c - other * sn : v[e] * c + other * sn;
-    }
-  }
+  norm_rotate_head<EPL>(v, lane, weight, eps, rotate ? inv_freq : nullptr,
+                        rotate ? static_cast<float>(positions[t]) : 0.f);
   if (dst != nullptr) {
 #pragma unroll
     for (int e = 0; e < EPL; ++e) dst[lane * EPL + e] = from_float<T>(v[e]);

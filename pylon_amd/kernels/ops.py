@@ -265,6 +265,57 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     return out
 
 
+def decode_fused_ok(qkv: torch.Tensor, k_cache: torch.Tensor, *, tokens: int, n_heads: int, head_dim: int,
+                    rot_dim: int) -> bool:
+    """Whether the decode kernel can prepare q, k and v itself: its geometry, and a rotation
+    of the whole head or none."""
+    n_kv_heads = k_cache.shape[2]
+    return (qkv.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and head_dim in DECODE_HEAD_DIMS
+            and tokens <= DECODE_MAX_TOKENS and n_heads % n_kv_heads == 0 and n_heads // n_kv_heads <= 16
+            and rot_dim in (0, head_dim) and qkv.stride(0) % 2 == 0 and qkv.stride(1) == 1)
+
+
+def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                           block_table: torch.Tensor, tok_row: Optional[torch.Tensor], positions: torch.Tensor, *,
+                           n_heads: int, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+                           eps: float, inv_freq: Optional[torch.Tensor], slot_map: Optional[torch.Tensor],
+                           page_size: int, window: Optional[int], scale: float, n_splits: int) -> torch.Tensor:
+    """:func:`qkv_prepare` and :func:`attention_decode` in one launch: from the raw projection
+    ``qkv`` ``[tokens, (n_heads + 2 kv_heads) * head_dim]`` (``[tokens, n_heads * head_dim]``
+    when ``slot_map`` is None and nothing is stored).  Returns ``[tokens, n_heads, head_dim]``."""
+    pages, psize, n_kv_heads, head_dim = k_cache.shape
+    tokens = qkv.shape[0]
+    store = slot_map is not None
+    if qkv.dim() != 2 or qkv.shape[1] != (n_heads + (2 * n_kv_heads if store else 0)) * head_dim:
+        raise KernelError("attention_decode_fused: the projection's width does not match the heads")
+    if not decode_fused_ok(qkv, k_cache, tokens=tokens, n_heads=n_heads, head_dim=head_dim,
+                           rot_dim=0 if inv_freq is None else 2 * inv_freq.numel()):
+        raise KernelError("attention_decode_fused does not take this geometry")
+    if psize != page_size or k_cache.shape != v_cache.shape or v_cache.dtype != k_cache.dtype:
+        raise KernelError("attention_decode_fused: cache geometry does not match page_size")
+    if pages * page_size >= 2 ** 31:
+        raise KernelError("attention_decode_fused: the cache holds more slots than an int32 can index")
+    if positions.numel() != tokens or block_table.dim() != 2 or (store and slot_map.numel() != tokens):
+        raise KernelError("attention_decode_fused: one position and one slot per token and a 2-D table are required")
+    for name, wt in (("q_weight", q_weight), ("k_weight", k_weight)):
+        if wt is not None and wt.shape != (head_dim,):
+            raise KernelError(f"attention_decode_fused: {name} must have shape ({head_dim},)")
+    if tok_row is None:
+        if block_table.shape[0] < tokens:
+            raise KernelError("attention_decode_fused: without row ids the table needs a row per token")
+    elif tok_row.numel() != tokens:
+        raise KernelError("attention_decode_fused: one row id per token is required")
+    out = torch.empty((tokens, n_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+    _lib.call("pylon_attention_decode_fused", _dev(out, "out"), qkv.data_ptr(), qkv.stride(0),
+              _dev(q_weight, "q_weight", torch.float32), _dev(k_weight, "k_weight", torch.float32), float(eps),
+              _dev(inv_freq, "inv_freq", torch.float32), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
+              _dev(slot_map, "slot_map", torch.int32), _dev(block_table, "block_table", torch.int32),
+              block_table.shape[1], _dev(tok_row, "tok_row", torch.int32),
+              _dev(positions, "positions", torch.int32), tokens, n_heads, n_kv_heads, head_dim, page_size,
+              int(window or 0), float(scale), int(n_splits), _stream())
+    return out
+
+
 PREFILL_ROWS = 64  # (token, head) query rows one workgroup of the prefill kernel takes
 
 
@@ -324,15 +375,25 @@ def gemm_tiled(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[tor
     return out
 
 
-# Most rows of x for which the weight-streaming kernel is chosen.  It takes up to 64, but
-# beyond one 16-row tile it re-reads x once per 16 weight rows, and the library's tiled
+# Most rows of x for which the first weight-streaming kernel is chosen.  It takes up to 64,
+# but beyond one 16-row tile it re-reads x once per 16 weight rows, and the library's tiled
 # kernels measured faster (e.g. 27 us against 64 us for the fused gate/up matrix at 64 rows).
+# A variant that stages x in LDS and shares it between four waves was tried for 17..64 rows:
+# it stayed behind the library too (43 us for that matrix), and where cutting K over
+# workgroups put it ahead (12 us against 19 us for a 2560 x 4096 matrix) the residual norm
+# paid the gain back by adding eight partial results of 64 rows.
 SKINNY_ROWS = 16
 
 
+def _streaming_ok(x: torch.Tensor, weight: torch.Tensor, rows: int) -> bool:
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < x.shape[0] <= rows
+            and weight.shape[1] % 8 == 0 and weight.stride(0) % 8 == 0 and x.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
 def skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < x.shape[0] <= SKINNY_ROWS
-            and weight.shape[1] % 8 == 0 and weight.stride(0) % 8 == 0 and x.stride(0) % 8 == 0)
+    """Few rows: the kernel whose waves split K and read x straight from memory."""
+    return _streaming_ok(x, weight, SKINNY_ROWS)
 
 
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype = torch.bfloat16,
@@ -376,7 +437,7 @@ def k_parts(n: int, k: int) -> int:
 def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """``x @ weight.T``.
 
-    bfloat16 by bfloat16: up to 64 rows go to the weight-streaming kernel, more rows to
+    bfloat16 by bfloat16: up to 16 rows go to the weight-streaming kernel, more rows to
     the library matrix product (as the reference's ``nn.Linear`` does).  Every pairing
     that involves float32 operands runs on the exact tiled kernel, which never uses a
     reduced-precision matrix mode.

@@ -49,8 +49,22 @@ class Attention(Part):
         if not stores:
             weight = weight[: spec.q_size]
         qkv = ops.linear(h, weight, out_dtype=self.dtype)
-        q = torch.empty((tokens, spec.n_heads, spec.head_dim), dtype=self.dtype, device=h.device)
         rotary = self.position.rotary()
+        if ctx.decode_only and cache.k is not None and ops.decode_fused_ok(
+                qkv, cache.k, tokens=tokens, n_heads=spec.n_heads, head_dim=spec.head_dim,
+                rot_dim=rotary[1] if rotary else 0):
+            # one launch norms and rotates q and k, stores k and v, and attends
+            splits = ops.decode_splits(tokens, spec.n_kv_heads, None if ctx.fixed_shapes else ctx.max_len)
+            context = ops.attention_decode_fused(
+                qkv, cache.k, cache.v, cache.block_table, None, ctx.positions,
+                n_heads=spec.n_heads, q_weight=self.params.get("q_norm"), k_weight=self.params.get("k_norm"),
+                eps=spec.qk_norm_eps, inv_freq=rotary[0] if rotary else None,
+                slot_map=cache.slot_map if stores else None,
+                page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits,
+            )
+            return ops.linear_for_residual(context.view(tokens, spec.q_size), self.params["out"],
+                                           out_dtype=self.dtype)
+        q = torch.empty((tokens, spec.n_heads, spec.head_dim), dtype=self.dtype, device=h.device)
         ops.qkv_prepare(
             qkv, q, cache.k, cache.v,
             n_heads=spec.n_heads, n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim,

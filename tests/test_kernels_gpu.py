@@ -607,6 +607,47 @@ def test_sampling_with_thousands_of_equal_logits_at_the_boundary(ops):
     _check_draws(ops, logits[1:2].repeat(3, 1), temps, torch.full((3,), 0.7), us, plain)
 
 
+@pytest.mark.parametrize("geom", [(8, 2, 128, True, True), (6, 6, 64, True, False), (5, 1, 256, False, True),
+                                  (16, 1, 64, True, True), (3, 3, 128, False, False)])
+@pytest.mark.parametrize("store", [True, False])
+def test_decode_attention_that_prepares_q_k_v_itself(ops, geom, store):
+    """One launch from the raw projection gives the bits of the two launches it replaces:
+    the prepared queries' attention output, and the key and value rows in the cache."""
+    nh, nkv, hd, normed, rotated = geom
+    page, pages, tokens, eps = 16, 40, 7, 3e-6
+    width = (nh + (2 * nkv if store else 0)) * hd
+    qkv = rnd((tokens, width), 51, torch.bfloat16).to(DEV)
+    qw = (1 + 0.2 * rnd((hd,), 52)).to(DEV) if normed else None
+    kw = (1 + 0.2 * rnd((hd,), 53)).to(DEV) if normed else None
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd))).to(DEV) if rotated else None
+    lengths = [1, 17, 64, 65, 200, 16, 333]  # the new token is the last of each
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32)
+    perm = torch.randperm(pages * 4, generator=torch.Generator().manual_seed(9)).to(torch.int32)
+    table = perm[: tokens * 21].reshape(tokens, 21) % (pages * 4)
+    # distinct pages per request so that no two tokens share a slot
+    table = torch.arange(tokens * 21, dtype=torch.int32).reshape(tokens, 21)
+    total_pages = tokens * 21
+    slots = torch.tensor([int(table[t, (n - 1) // page]) * page + (n - 1) % page for t, n in enumerate(lengths)],
+                         dtype=torch.int32)
+    kc = (rnd((total_pages, page, nkv, hd), 54, torch.bfloat16) * 0.5).to(DEV)
+    vc = rnd((total_pages, page, nkv, hd), 55, torch.bfloat16).to(DEV)
+    kc2, vc2 = kc.clone(), vc.clone()
+    for window in (None, 50):
+        for splits in (1, 4, 8):
+            q = torch.empty((tokens, nh, hd), dtype=torch.bfloat16, device=DEV)
+            ops.qkv_prepare(qkv, q, kc, vc, n_heads=nh, n_kv_heads=nkv, head_dim=hd, q_weight=qw, k_weight=kw,
+                            eps=eps, inv_freq=inv_freq, rot_dim=hd if rotated else 0,
+                            positions=positions.to(DEV), slot_map=slots.to(DEV), store_kv=store)
+            want = ops.attention_decode(q, kc, vc, table.to(DEV), None, positions.to(DEV), page_size=page,
+                                        window=window, scale=hd ** -0.5, n_splits=splits)
+            got = ops.attention_decode_fused(
+                qkv, kc2, vc2, table.to(DEV), None, positions.to(DEV), n_heads=nh, q_weight=qw, k_weight=kw,
+                eps=eps, inv_freq=inv_freq, slot_map=slots.to(DEV) if store else None, page_size=page,
+                window=window, scale=hd ** -0.5, n_splits=splits)
+            assert torch.equal(got, want), (window, splits)
+            assert torch.equal(kc2, kc) and torch.equal(vc2, vc)
+
+
 def test_kernels_refuse_what_they_cannot_do(ops):
     from pylon_amd.kernels import KernelError
 
