@@ -98,24 +98,46 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
   if (k_end > pos + 1) k_end = pos + 1;
 
   if constexpr (PREP) {
-    // One wave per head: the group's query heads into LDS, then this key head and this
-    // value head into the token's cache slot.
+    // 512/head_dim heads per wave at a time: the group's query heads into LDS, then this
+    // key head and this value head into the token's cache slot.
+    constexpr int LPH = HD / 8, HPW = PYLON_WAVE / LPH;
+    // the token's rotation table, one private copy per wave: no workgroup barrier before use
+    float* cs = reinterpret_cast<float*>(q_lds + GP * HD) + wave * HD;
     const uint16_t* row = prep.qkv + static_cast<size_t>(t) * prep.row_stride;
     const int slot = prep.slot_map != nullptr ? prep.slot_map[t] : -1;
     const int jobs = group + (slot >= 0 ? 2 : 0);
-    const float fpos = static_cast<float>(pos);
-    for (int job = wave; job < jobs; job += n_waves) {
-      float v[EPL];
-      if (job < group) {
-        load_head_bf16<EPL>(row + static_cast<size_t>(kvh * group + job) * HD, lane, v);
-        norm_rotate_head<EPL>(v, lane, prep.q_weight, prep.eps, prep.inv_freq, fpos);
-        store_head_bf16<EPL>(q_lds + job * HD, lane, v);
-      } else {
-        const bool is_key = job == group;
-        load_head_bf16<EPL>(row + static_cast<size_t>(n_heads + (is_key ? 0 : n_kv_heads) + kvh) * HD, lane, v);
-        if (is_key) norm_rotate_head<EPL>(v, lane, prep.k_weight, prep.eps, prep.inv_freq, fpos);
-        uint16_t* dst = (is_key ? k_cache : v_cache) + (static_cast<size_t>(slot) * n_kv_heads + kvh) * HD;
-        store_head_bf16<EPL>(dst, lane, v);
+    const int j = lane % LPH;
+    // job -> where its head lies in the projection's row
+    auto source = [&](int job) {
+      const int head = job < group ? kvh * group + job : n_heads + (job == group ? 0 : n_kv_heads) + kvh;
+      return row + static_cast<size_t>(head) * HD + 8 * j;
+    };
+    // The first round's loads do not wait for the position.
+    int job = wave * HPW + lane / LPH;
+    float v[8];
+    load8_bf16(source(job < jobs ? job : jobs - 1), v);
+    if (prep.inv_freq != nullptr && wave * HPW < jobs) {
+      const float fpos = static_cast<float>(pos);
+      for (int i = lane; i < HD / 2; i += PYLON_WAVE) {
+        const float angle = fpos * prep.inv_freq[i];
+        cs[i] = cosf(angle);
+        cs[HD / 2 + i] = sinf(angle);
+      }
+      __builtin_amdgcn_wave_barrier();  // private to the wave: program order suffices
+    }
+    for (int h0 = wave * HPW; h0 < jobs; h0 += n_waves * HPW) {
+      job = h0 + lane / LPH;
+      const bool valid = job < jobs;
+      if (!valid) job = jobs - 1;
+      if (h0 != wave * HPW) load8_bf16(source(job), v);
+      const bool is_q = job < group, is_key = job == group;
+      const float* weight = is_q ? prep.q_weight : (is_key ? prep.k_weight : nullptr);
+      norm_rotate8<HD>(v, j, weight, prep.eps, (prep.inv_freq != nullptr && (is_q || is_key)) ? cs : nullptr);
+      if (valid && is_q) {
+        store8_bf16(q_lds + job * HD + 8 * j, v);
+      } else if (valid) {
+        uint16_t* dst = (is_key ? k_cache : v_cache) + (static_cast<size_t>(slot) * n_kv_heads + kvh) * HD + 8 * j;
+        store8_bf16(dst, v);
       }
     }
     // The barrier orders the workgroup's stores before its loads: every wave sees the new
@@ -285,7 +307,7 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
 
 static size_t decode_lds_bytes(int n_waves, int gp, int head_dim, bool prep) {
   return sizeof(float) * decode_lds_floats(n_waves, gp, head_dim) +
-         (prep ? sizeof(uint16_t) * static_cast<size_t>(gp) * head_dim : 0);
+         (prep ? sizeof(uint16_t) * static_cast<size_t>(gp) * head_dim + sizeof(float) * n_waves * head_dim : 0);
 }
 
 template <int EPL, bool PREP>
@@ -373,8 +395,8 @@ extern "C" int pylon_attention_decode_fused(void* out, const void* qkv, long lon
   const long long heads = n_heads + (slot_map != nullptr ? 2ll * n_kv_heads : 0);
   PYLON_REQUIRE(row_stride >= heads * head_dim, "attention_decode_fused: row stride %lld is shorter than %lld heads of %d",
                 row_stride, heads, head_dim);
-  PYLON_REQUIRE(row_stride % 2 == 0 && (reinterpret_cast<uintptr_t>(qkv) & 3) == 0,
-                "attention_decode_fused: the projection's rows must be 4-byte aligned");
+  PYLON_REQUIRE(row_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(qkv) & 15) == 0,
+                "attention_decode_fused: the projection's rows must be 16-byte aligned");
   if (tokens == 0) return 0;
   const DecodePrep prep = {static_cast<const uint16_t*>(qkv), row_stride, q_weight, k_weight, eps, inv_freq, slot_map};
 #define GO(D)                                                                                            \

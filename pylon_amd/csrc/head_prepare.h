@@ -59,3 +59,67 @@ __device__ __forceinline__ void store_head_bf16(uint16_t* __restrict__ dst, int 
     }
   }
 }
+
+// ---- the same for bfloat16 with 16-byte accesses -----------------------------------------
+// head_dim/8 lanes share a head, 8 consecutive elements each, so a wavefront prepares
+// 512/head_dim heads at once.  j is the lane's index within its head (lane % (HD/8)).
+// Every lane of the wave must call these together (they exchange values inside a head).
+
+// cos(pos * f_i) and sin(pos * f_i) for the HD/2 rotation pairs of one token, by the whole
+// workgroup: cs[i] and cs[HD/2 + i].  A barrier must follow before cs is read.
+template <int HD>
+__device__ __forceinline__ void rotation_table(float* __restrict__ cs, const float* __restrict__ inv_freq, float pos) {
+  for (int i = threadIdx.x; i < HD / 2; i += blockDim.x) {
+    const float angle = pos * inv_freq[i];
+    cs[i] = cosf(angle);
+    cs[HD / 2 + i] = sinf(angle);
+  }
+}
+
+__device__ __forceinline__ void load8_bf16(const uint16_t* __restrict__ src, float v[8]) {
+  const uint4 raw = *reinterpret_cast<const uint4*>(src);
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __uint_as_float(w[i] << 16);
+    v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
+__device__ __forceinline__ void store8_bf16(uint16_t* __restrict__ dst, const float v[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    w[i] = static_cast<uint32_t>(float_to_bf16_bits(v[2 * i])) |
+           (static_cast<uint32_t>(float_to_bf16_bits(v[2 * i + 1])) << 16);
+  *reinterpret_cast<uint4*>(dst) = uint4{w[0], w[1], w[2], w[3]};
+}
+
+// v: elements 8j .. 8j+7 of a head.  weight: the head's RMSNorm weight or null (per lane:
+// heads in one wave may differ).  cs: the token's rotation table or null.
+template <int HD>
+__device__ __forceinline__ void norm_rotate8(float v[8], int j, const float* __restrict__ weight, float eps,
+                                             const float* __restrict__ cs) {
+  constexpr int LPH = HD / 8;
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
+#pragma unroll
+  for (int off = 1; off < LPH; off <<= 1) ss += __shfl_xor(ss, off, PYLON_WAVE);
+  if (weight != nullptr) {
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(HD) + eps);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (v[e] * inv) * weight[8 * j + e];
+  }
+  const bool rotate = cs != nullptr;
+  const bool low = j < LPH / 2;
+  const int pair0 = 8 * (j & (LPH / 2 - 1));
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float other = __shfl_xor(v[e], LPH / 2, PYLON_WAVE);
+    if (rotate) {
+      const float c = cs[pair0 + e], sn = cs[HD / 2 + pair0 + e];
+      v[e] = low ? v[e] * c - other * sn : v[e] * c + other * sn;
+    }
+  }
+}

@@ -149,6 +149,81 @@ __global__ void qkv_prepare_wide_kernel(T* __restrict__ q_out, T* __restrict__ k
   }
 }
 
+// bfloat16 at head sizes 64/128/256 with the whole head rotated (or none of it): a
+// workgroup takes a share of one token's heads.  The token's rotation table is computed once
+// into LDS; then each wave prepares 512/head_dim heads at a time with 16-byte accesses.
+template <int HD>
+__global__ __launch_bounds__(QKV_WAVES* PYLON_WAVE) void qkv_prepare_rows_kernel(
+    uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache,
+    const uint16_t* __restrict__ qkv, long long row_stride, const float* __restrict__ q_weight,
+    const float* __restrict__ k_weight, float eps, const float* __restrict__ inv_freq,
+    const int* __restrict__ positions, const int* __restrict__ slot_map, int n_heads, int n_kv_heads,
+    int heads_per_token, int heads_per_block) {
+  constexpr int LPH = HD / 8, HPW = PYLON_WAVE / LPH;
+  __shared__ float cs[HD];
+  const int lane = threadIdx.x & (PYLON_WAVE - 1);
+  const int wave = threadIdx.x / PYLON_WAVE;
+  const int t = blockIdx.x;
+  if (inv_freq != nullptr) {
+    rotation_table<HD>(cs, inv_freq, static_cast<float>(positions[t]));
+    __syncthreads();
+  }
+  const int h_begin = blockIdx.y * heads_per_block;
+  const int h_end = h_begin + heads_per_block < heads_per_token ? h_begin + heads_per_block : heads_per_token;
+  const int slot = heads_per_token > n_heads ? slot_map[t] : -1;
+  const uint16_t* row = qkv + static_cast<size_t>(t) * row_stride;
+  const int j = lane % LPH;
+  for (int h0 = h_begin + wave * HPW; h0 < h_end; h0 += QKV_WAVES * HPW) {
+    const int mine = h0 + lane / LPH;
+    const bool valid = mine < h_end;
+    const int s = valid ? mine : h_end - 1;
+    const uint16_t* src = row + static_cast<size_t>(s) * HD + 8 * j;  // heads lie in the order q, k, v
+    uint16_t* dst = nullptr;
+    const float* weight = nullptr;
+    bool rotate = false;
+    if (s < n_heads) {
+      dst = q_out + (static_cast<size_t>(t) * n_heads + s) * HD + 8 * j;
+      weight = q_weight;
+      rotate = true;
+    } else {
+      const bool is_key = s - n_heads < n_kv_heads;
+      const int kvh = is_key ? s - n_heads : s - n_heads - n_kv_heads;
+      if (slot >= 0) dst = (is_key ? k_cache : v_cache) + (static_cast<size_t>(slot) * n_kv_heads + kvh) * HD + 8 * j;
+      weight = is_key ? k_weight : nullptr;
+      rotate = is_key;
+    }
+    float v[8];
+    load8_bf16(src, v);
+    norm_rotate8<HD>(v, j, weight, eps, (rotate && inv_freq != nullptr) ? cs : nullptr);
+    if (valid && dst != nullptr) store8_bf16(dst, v);
+  }
+}
+
+static bool launch_rows(uint16_t* q_out, uint16_t* k_cache, uint16_t* v_cache, const uint16_t* qkv,
+                        long long row_stride, const float* q_weight, const float* k_weight, float eps,
+                        const float* inv_freq, const int* positions, const int* slot_map, int tokens,
+                        int n_heads, int n_kv_heads, int head_dim, int heads_per_token, hipStream_t stream) {
+  // enough workgroups to fill the chip when there are few tokens
+  const int per_round = QKV_WAVES * (512 / head_dim);  // heads a workgroup prepares at a time
+  int shares = 1;
+  while (tokens * shares < 1024 && shares * per_round < heads_per_token) shares *= 2;
+  int heads_per_block = (heads_per_token + shares - 1) / shares;
+  heads_per_block = (heads_per_block + per_round - 1) / per_round * per_round;
+  shares = (heads_per_token + heads_per_block - 1) / heads_per_block;
+  dim3 grid(tokens, shares), block(QKV_WAVES * PYLON_WAVE);
+#define GO(HD)                                                                                          \
+  hipLaunchKernelGGL((qkv_prepare_rows_kernel<HD>), grid, block, 0, stream, q_out, k_cache, v_cache, qkv, \
+                     row_stride, q_weight, k_weight, eps, inv_freq, positions, slot_map, n_heads,       \
+                     n_kv_heads, heads_per_token, heads_per_block)
+  switch (head_dim) {
+    case 64: GO(64); return true;
+    case 128: GO(128); return true;
+    case 256: GO(256); return true;
+    default: return false;
+  }
+#undef GO
+}
+
 template <typename T>
 static bool launch_wide(T* q_out, T* k_cache, T* v_cache, const T* qkv, long long row_stride,
                         const float* q_weight, const float* k_weight, float eps, const float* inv_freq,
@@ -198,7 +273,14 @@ extern "C" int pylon_qkv_prepare(void* q_out, void* k_cache, void* v_cache, cons
   // whole-head rotation (or none) at head sizes 64/128/256 takes the vector form
   if ((inv_freq == nullptr || rot_dim == head_dim) && row_stride % 2 == 0) {
     bool done;
-    if (dtype == PYLON_F32)
+    const bool vectors = dtype == PYLON_BF16 && row_stride % 8 == 0 &&
+                         (reinterpret_cast<uintptr_t>(qkv) & 15) == 0 &&
+                         (reinterpret_cast<uintptr_t>(q_out) & 15) == 0;
+    if (vectors)
+      done = launch_rows((uint16_t*)q_out, (uint16_t*)k_cache, (uint16_t*)v_cache, (const uint16_t*)qkv,
+                         row_stride, q_weight, k_weight, eps, inv_freq, positions, slot_map, tokens, n_heads,
+                         n_kv_heads, head_dim, heads_per_token, stream);
+    else if (dtype == PYLON_F32)
       done = launch_wide<float>((float*)q_out, (float*)k_cache, (float*)v_cache, (const float*)qkv, row_stride,
                                 q_weight, k_weight, eps, inv_freq, positions, slot_map, items, n_heads,
                                 n_kv_heads, head_dim, heads_per_token, grid, block, stream);

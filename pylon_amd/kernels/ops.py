@@ -272,7 +272,8 @@ def decode_fused_ok(qkv: torch.Tensor, k_cache: torch.Tensor, *, tokens: int, n_
     n_kv_heads = k_cache.shape[2]
     return (qkv.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and head_dim in DECODE_HEAD_DIMS
             and tokens <= DECODE_MAX_TOKENS and n_heads % n_kv_heads == 0 and n_heads // n_kv_heads <= 16
-            and rot_dim in (0, head_dim) and qkv.stride(0) % 2 == 0 and qkv.stride(1) == 1)
+            and rot_dim in (0, head_dim) and qkv.stride(0) % 8 == 0 and qkv.stride(1) == 1
+            and qkv.data_ptr() % 16 == 0)
 
 
 def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
