@@ -3,29 +3,41 @@
 //
 // A workgroup of four wavefronts takes one tile of consecutive tokens of one request and
 // one key/value head, together with all query heads of that head's group: a (token, head)
-// pair is one of up to 64 query rows, 16 per wave.  Keys and values are walked 64 at a
-// time.  The workgroup stages the 64 keys (row-major) and the 64 values (transposed, so
-// that a lane can read four consecutive keys of one element) in LDS.  Scores are computed
-// transposed (keys as rows, queries as columns): the result registers of a score tile then
-// already have the layout the row operand of the value product needs, and the running
-// maximum and sum of a query live in the lanes of its column.  Scores, softmax and the
-// output accumulators are float.
+// pair is one of up to 64 or 128 query rows, 16 or 32 per wave.  Keys and values are walked
+// 64 at a time.  While one block of keys is being used, the next is already on its way
+// from the cache into registers; at the top of an iteration the registers go to LDS: the
+// 64 keys row-major, the 64 values transposed (a thread holds eight elements of four
+// consecutive keys and writes, per element, the four keys as one 8-byte word), so that a
+// lane reads the column operand of the value product as two 8-byte words.  Scores are
+// computed transposed (keys as rows, queries as columns): the result registers of a score
+// tile then already have the layout the row operand of the value product needs, and the
+// running maximum and sum of a query live in the lanes of its column.  Scores, softmax and
+// the output accumulators are float; exponentials are exp2 with scale*log2(e) folded into
+// one multiply-add.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 #define AP_BK 64       // keys per iteration
-#define AP_ROWS 64     // query rows per workgroup
-#define AP_QT 1        // 16-row query tiles per wave
-#define AP_VSTRIDE 66  // keys per row of the transposed value tile (+2: spreads LDS banks)
+#define AP_VSTRIDE 68  // keys per row of the transposed value tile (136 bytes: 8-byte aligned rows)
+#define AP_SLACK 8.0f  // how far (as a power of two) a score may exceed the maximum in use
+#define AP_TABLE 4096  // most pages a request may hold: its block-table row is kept in LDS
 
+// Two floats to two bfloat16 (round to nearest even) in one word: the hardware conversion.
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  return static_cast<uint32_t>(float_to_bf16_bits(lo)) | (static_cast<uint32_t>(float_to_bf16_bits(hi)) << 16);
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{lo, hi}, bf16x2));
 }
 
-template <int HD>
-__global__ __launch_bounds__(256) void attention_prefill_kernel(
+// QT: 16-row query tiles per wave (1: 64 rows per workgroup, 2: 128).  POW2: the page size
+// is a power of two, so a key's page and offset are a shift and a mask (a division by a
+// run-time number costs some twenty instructions, eight times per thread and block).
+template <int HD, int QT, bool POW2>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) void attention_prefill_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, int n_heads, int n_kv_heads, int group, int page_size, int window,
@@ -33,9 +45,12 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   constexpr int KS = HD / 32;        // 32-wide steps along the head for a score tile
   constexpr int DT = HD / 16;        // 16-wide output tiles along the head
   constexpr int KSTR = HD + 8;       // row stride of the key tile (elements)
-  constexpr int CHUNKS = HD / 8;     // 16-byte chunks per key row
+  constexpr int CHUNKS = HD / 8;     // 16-byte chunks per key or value row
+  constexpr int KP = AP_BK * CHUNKS / 256;          // 16-byte pieces of keys per thread and block
+  constexpr int VC = (CHUNKS * 16 + 255) / 256;     // (chunk, four keys) items of values per thread
   __shared__ __attribute__((aligned(16))) uint16_t k_lds[AP_BK * KSTR];
   __shared__ __attribute__((aligned(16))) uint16_t v_lds[HD * AP_VSTRIDE];
+  __shared__ int table_lds[AP_TABLE];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -44,13 +59,61 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   const int* td = tiles + blockIdx.x * 4;
   const int tok0 = td[0], ntok = td[1], trow = td[2], pos0 = td[3];
   const int* table = block_table + static_cast<size_t>(trow) * table_width;
+  const int kv_last = pos0 + ntok - 1;
+  const int k_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int kb_first = (k_lo / AP_BK) * AP_BK;
+  // The request's page ids go to LDS once, so that finding a key's page costs no trip to
+  // memory inside the loop (the host refuses requests with more pages than fit).
+  const int pages_used = kv_last / page_size + 1;
+  for (int i = tid; i < pages_used; i += 256) table_lds[i] = table[i];
+  __syncthreads();
+
+  // The block of keys and values on its way from the cache.  Keys: piece i of a thread is
+  // 8 elements of key (i*256 + tid) / CHUNKS.  Values: item i is chunk (i*256 + tid) / 16
+  // of keys 4*((i*256 + tid) % 16) .. +3.  Keys past the end repeat the last key.
+  u32x4 kreg[KP], vreg[VC][4];
+  const int page_shift = __ffs(page_size) - 1, page_mask = page_size - 1;
+  const size_t row_elems = static_cast<size_t>(n_kv_heads) * HD;
+  const uint16_t* k_head = k_cache + static_cast<size_t>(kvh) * HD;
+  const uint16_t* v_head = v_cache + static_cast<size_t>(kvh) * HD;
+#define AP_SLOT(J, PHYS)                                                                               \
+  do {                                                                                                 \
+    const int pg = POW2 ? (J) >> page_shift : (J) / page_size;                                         \
+    const int off = POW2 ? (J) & page_mask : (J) - pg * page_size;                                     \
+    PHYS = table_lds[pg] * page_size + off;                                                            \
+  } while (0)
+#define AP_FETCH(KB)                                                                                   \
+  do {                                                                                                 \
+    _Pragma("unroll") for (int i = 0; i < KP; ++i) {                                                   \
+      const int idx = i * 256 + tid;                                                                   \
+      const int key = idx / CHUNKS, chunk = idx - key * CHUNKS;                                        \
+      const int j = ((KB) + key < kv_last) ? (KB) + key : kv_last;                                     \
+      int phys;                                                                                        \
+      AP_SLOT(j, phys);                                                                                \
+      kreg[i] = *reinterpret_cast<const u32x4*>(k_head + static_cast<size_t>(phys) * row_elems + chunk * 8); \
+    }                                                                                                  \
+    _Pragma("unroll") for (int i = 0; i < VC; ++i) {                                                   \
+      const int idx = i * 256 + tid;                                                                   \
+      const int chunk = idx >> 4, quad = idx & 15;                                                     \
+      if (chunk < CHUNKS) {                                                                            \
+        _Pragma("unroll") for (int p = 0; p < 4; ++p) {                                                \
+          const int j = ((KB) + 4 * quad + p < kv_last) ? (KB) + 4 * quad + p : kv_last;               \
+          int phys;                                                                                    \
+          AP_SLOT(j, phys);                                                                            \
+          vreg[i][p] = *reinterpret_cast<const u32x4*>(v_head + static_cast<size_t>(phys) * row_elems + chunk * 8); \
+        }                                                                                              \
+      }                                                                                                \
+    }                                                                                                  \
+  } while (0)
+
+  AP_FETCH(kb_first);
 
   // this lane's query column in each of the wave's query tiles
-  int qpos[AP_QT];
-  bf16x8 qf[AP_QT][KS];
+  int qpos[QT];
+  bf16x8 qf[QT][KS];
 #pragma unroll
-  for (int qt = 0; qt < AP_QT; ++qt) {
-    const int rr = wave * (16 * AP_QT) + qt * 16 + col;
+  for (int qt = 0; qt < QT; ++qt) {
+    const int rr = wave * (16 * QT) + qt * 16 + col;
     const int ti = rr / group, hh = rr - ti * group;
     const bool valid = ti < ntok;
     qpos[qt] = valid ? pos0 + ti : -1;
@@ -66,10 +129,10 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     }
   }
 
-  float m_run[AP_QT], l_run[AP_QT];
-  floatx4 o[AP_QT][DT];
+  float m_run[QT], l_run[QT];  // the running maximum is kept in units of raw scores
+  floatx4 o[QT][DT];
 #pragma unroll
-  for (int qt = 0; qt < AP_QT; ++qt) {
+  for (int qt = 0; qt < QT; ++qt) {
     m_run[qt] = -INFINITY;
     l_run[qt] = 0.f;
 #pragma unroll
@@ -77,98 +140,110 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   }
 
   const float scale_log2 = scale * 1.44269504088896340736f;
-  const int kv_last = pos0 + ntok - 1;
-  const int k_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
-  for (int kb = (k_lo / AP_BK) * AP_BK; kb <= kv_last; kb += AP_BK) {
-    __syncthreads();
-    // stage 64 keys row-major and 64 values transposed
+  const float slack = AP_SLACK / scale_log2;  // in units of raw scores
+  for (int kb = kb_first; kb <= kv_last; kb += AP_BK) {
+    __syncthreads();  // the last block's readers are done
+    // registers -> LDS: keys row-major, values transposed
 #pragma unroll
-    for (int pass = 0; pass < AP_BK * CHUNKS / 256; ++pass) {
-      const int idx = pass * 256 + tid;
+    for (int i = 0; i < KP; ++i) {
+      const int idx = i * 256 + tid;
       const int key = idx / CHUNKS, chunk = idx - key * CHUNKS;
-      const int j = (kb + key < kv_last) ? kb + key : kv_last;  // past the end: repeat the last key
-      const int phys = table[j / page_size] * page_size + j % page_size;
-      const size_t src = (static_cast<size_t>(phys) * n_kv_heads + kvh) * HD + chunk * 8;
-      const uint4 kvec = *reinterpret_cast<const uint4*>(k_cache + src);
-      const uint4 vvec = *reinterpret_cast<const uint4*>(v_cache + src);
-      *reinterpret_cast<uint4*>(&k_lds[key * KSTR + chunk * 8]) = kvec;
-      const uint32_t vw[4] = {vvec.x, vvec.y, vvec.z, vvec.w};
+      *reinterpret_cast<u32x4*>(&k_lds[key * KSTR + chunk * 8]) = kreg[i];
+    }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        v_lds[(chunk * 8 + 2 * i) * AP_VSTRIDE + key] = static_cast<uint16_t>(vw[i] & 0xffffu);
-        v_lds[(chunk * 8 + 2 * i + 1) * AP_VSTRIDE + key] = static_cast<uint16_t>(vw[i] >> 16);
+    for (int i = 0; i < VC; ++i) {
+      const int idx = i * 256 + tid;
+      const int chunk = idx >> 4, quad = idx & 15;
+      if (chunk < CHUNKS) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {  // elements chunk*8 + 2e and + 2e + 1 of the four keys
+          const uint32_t w0 = vreg[i][0][e], w1 = vreg[i][1][e], w2 = vreg[i][2][e], w3 = vreg[i][3][e];
+          // byte selects: the low halves of two words side by side, and the high halves
+          const u32x2 even = {__builtin_amdgcn_perm(w1, w0, 0x05040100u), __builtin_amdgcn_perm(w3, w2, 0x05040100u)};
+          const u32x2 odd = {__builtin_amdgcn_perm(w1, w0, 0x07060302u), __builtin_amdgcn_perm(w3, w2, 0x07060302u)};
+          *reinterpret_cast<u32x2*>(&v_lds[(chunk * 8 + 2 * e) * AP_VSTRIDE + 4 * quad]) = even;
+          *reinterpret_cast<u32x2*>(&v_lds[(chunk * 8 + 2 * e + 1) * AP_VSTRIDE + 4 * quad]) = odd;
+        }
       }
     }
+    if (kb + AP_BK <= kv_last) AP_FETCH(kb + AP_BK);  // the next block travels during this one's math
     __syncthreads();
 
     // transposed scores: rows = keys of a 16-key tile, columns = the query tile's rows
-    floatx4 s[AP_QT][AP_BK / 16];
-#pragma unroll
-    for (int qt = 0; qt < AP_QT; ++qt)
-#pragma unroll
-      for (int kt = 0; kt < AP_BK / 16; ++kt) s[qt][kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    floatx4 s[QT][AP_BK / 16];
 #pragma unroll
     for (int kt = 0; kt < AP_BK / 16; ++kt) {
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&k_lds[(kt * 16 + col) * KSTR + ks * 32 + grp * 8]);
 #pragma unroll
-        for (int qt = 0; qt < AP_QT; ++qt)
-          s[qt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qt][ks], s[qt][kt], 0, 0, 0);
+        for (int qt = 0; qt < QT; ++qt)
+          s[qt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              kf, qf[qt][ks], ks == 0 ? floatx4{0.f, 0.f, 0.f, 0.f} : s[qt][kt], 0, 0, 0);
       }
     }
 
-    // mask, running softmax, and the probabilities as row operands of the value product.
-    // Scores are scaled by scale*log2(e) so that the exponentials are single exp2
-    // instructions; the running maximum is kept in the same units.
-    bf16x8 pa[AP_QT][AP_BK / 32];
+    // mask (only blocks that reach past the tile's first query, or a window's edge, need
+    // it), running softmax, and the probabilities as row operands of the value product
+    const bool masked = kb + AP_BK - 1 > pos0 || window > 0;
+    bf16x8 pa[QT][AP_BK / 32];
 #pragma unroll
-    for (int qt = 0; qt < AP_QT; ++qt) {
-      const int qp = qpos[qt];
-      const int lo = (window > 0) ? qp - window + 1 : 0;
+    for (int qt = 0; qt < QT; ++qt) {
+      if (masked) {
+        const int qp = qpos[qt];
+        const int lo = (window > 0) ? qp - window + 1 : 0;
+#pragma unroll
+        for (int kt = 0; kt < AP_BK / 16; ++kt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int key = kb + kt * 16 + 4 * grp + r;
+            if (!(key <= qp && key >= lo)) s[qt][kt][r] = -INFINITY;
+          }
+      } else if (qpos[qt] < 0) {  // a column that holds no query
+#pragma unroll
+        for (int kt = 0; kt < AP_BK / 16; ++kt) s[qt][kt] = floatx4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+      }
+      // The maximum that the exponentials are taken against is raised only when a score
+      // exceeds it by more than AP_SLACK (in units of exp2's argument): until then
+      // probabilities may reach 2^AP_SLACK instead of 1, which float sums and bfloat16
+      // operands hold just as well, and neither the cross-lane maximum nor the rescaling
+      // of the accumulators is needed.  The result is the same up to rounding.
       float tile_max = -INFINITY;
 #pragma unroll
       for (int kt = 0; kt < AP_BK / 16; ++kt)
 #pragma unroll
+        for (int r = 0; r < 4; ++r) tile_max = fmaxf(tile_max, s[qt][kt][r]);
+      if (__ballot(tile_max > m_run[qt] + slack) != 0) {  // the same for the whole wave
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, PYLON_WAVE));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, PYLON_WAVE));
+        const float m_new = fmaxf(m_run[qt], tile_max);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen no key yet
+        const float corr = __builtin_amdgcn_exp2f((m_run[qt] - m_use) * scale_log2);
+        l_run[qt] *= corr;
+        m_run[qt] = m_new;
+        // the accumulators of this lane belong to query rows 4*grp + r: fetch their factors
+#pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int key = kb + kt * 16 + 4 * grp + r;
-          const float v = (key <= qp && key >= lo) ? s[qt][kt][r] * scale_log2 : -INFINITY;
-          s[qt][kt][r] = v;
-          tile_max = fmaxf(tile_max, v);
+          const float c = __shfl(corr, 4 * grp + r, PYLON_WAVE);
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) o[qt][dt][r] *= c;
         }
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, PYLON_WAVE));
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, PYLON_WAVE));
-      const float m_new = fmaxf(m_run[qt], tile_max);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen no key yet
-      const float corr = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
-      float tile_sum = 0.f;
+      }
+      const float shift = (m_run[qt] == -INFINITY) ? 0.f : -m_run[qt] * scale_log2;
       float p[AP_BK / 16][4];
 #pragma unroll
       for (int kt = 0; kt < AP_BK / 16; ++kt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          p[kt][r] = __builtin_amdgcn_exp2f(s[qt][kt][r] - m_use);
-          tile_sum += p[kt][r];
+          p[kt][r] = __builtin_amdgcn_exp2f(fmaf(s[qt][kt][r], scale_log2, shift));
+          l_run[qt] += p[kt][r];  // this lane's share of the row's sum; the lanes meet at the end
         }
-      tile_sum += __shfl_xor(tile_sum, 16, PYLON_WAVE);
-      tile_sum += __shfl_xor(tile_sum, 32, PYLON_WAVE);
-      l_run[qt] = l_run[qt] * corr + tile_sum;
-      m_run[qt] = m_new;
 #pragma unroll
       for (int kg = 0; kg < AP_BK / 32; ++kg) {
-        uint4 packed;
-        packed.x = pack_bf16(p[2 * kg][0], p[2 * kg][1]);
-        packed.y = pack_bf16(p[2 * kg][2], p[2 * kg][3]);
-        packed.z = pack_bf16(p[2 * kg + 1][0], p[2 * kg + 1][1]);
-        packed.w = pack_bf16(p[2 * kg + 1][2], p[2 * kg + 1][3]);
-        pa[qt][kg] = *reinterpret_cast<bf16x8*>(&packed);
-      }
-      // the accumulators of this lane belong to query rows 4*grp + r: fetch their factors
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float c = __shfl(corr, 4 * grp + r, PYLON_WAVE);
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) o[qt][dt][r] *= c;
+        const u32x4 packed = {pack_bf16(p[2 * kg][0], p[2 * kg][1]), pack_bf16(p[2 * kg][2], p[2 * kg][3]),
+                              pack_bf16(p[2 * kg + 1][0], p[2 * kg + 1][1]),
+                              pack_bf16(p[2 * kg + 1][2], p[2 * kg + 1][3])};
+        pa[qt][kg] = __builtin_bit_cast(bf16x8, packed);
       }
     }
 
@@ -179,26 +254,29 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
         const uint16_t* vrow = &v_lds[(dt * 16 + col) * AP_VSTRIDE + kg * 32 + 4 * grp];
-        uint4 vv;
-        vv.x = *reinterpret_cast<const uint32_t*>(vrow);
-        vv.y = *reinterpret_cast<const uint32_t*>(vrow + 2);
-        vv.z = *reinterpret_cast<const uint32_t*>(vrow + 16);
-        vv.w = *reinterpret_cast<const uint32_t*>(vrow + 18);
-        const bf16x8 vf = *reinterpret_cast<bf16x8*>(&vv);
+        const u32x2 first = *reinterpret_cast<const u32x2*>(vrow);
+        const u32x2 second = *reinterpret_cast<const u32x2*>(vrow + 16);
+        const u32x4 vv = {first[0], first[1], second[0], second[1]};
+        const bf16x8 vf = __builtin_bit_cast(bf16x8, vv);
 #pragma unroll
-        for (int qt = 0; qt < AP_QT; ++qt)
+        for (int qt = 0; qt < QT; ++qt)
           o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[qt][kg], vf, o[qt][dt], 0, 0, 0);
       }
     }
   }
+#undef AP_FETCH
+#undef AP_SLOT
 
   // out = acc / sum; this lane holds rows 4*grp + r, element dt*16 + col
 #pragma unroll
-  for (int qt = 0; qt < AP_QT; ++qt) {
+  for (int qt = 0; qt < QT; ++qt) {
+    float l_row = l_run[qt];  // the four lanes of a query column each hold a share
+    l_row += __shfl_xor(l_row, 16, PYLON_WAVE);
+    l_row += __shfl_xor(l_row, 32, PYLON_WAVE);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const float l = __shfl(l_run[qt], 4 * grp + r, PYLON_WAVE);
-      const int rr = wave * (16 * AP_QT) + qt * 16 + 4 * grp + r;
+      const float l = __shfl(l_row, 4 * grp + r, PYLON_WAVE);
+      const int rr = wave * (16 * QT) + qt * 16 + 4 * grp + r;
       const int ti = rr / group, hh = rr - ti * group;
       if (ti < ntok) {
         const float inv = 1.0f / l;
@@ -212,33 +290,48 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 
 // tiles: [n_tiles, 4] = (index of the tile's first token in q/out, its token count, its row of
 // the block table, the position of its first token).  A tile holds consecutive tokens of one
-// request, at most floor(64 / group) of them.
+// request, at most floor(rows / group) of them; rows (64 or 128) is the number of (token,
+// head) query rows a workgroup takes.
 extern "C" int pylon_attention_prefill(void* out, const void* q, const void* k_cache, const void* v_cache,
                                        const int* block_table, int table_width, const int* tiles,
                                        int n_tiles, int n_heads, int n_kv_heads, int head_dim,
-                                       int page_size, int window, float scale, hipStream_t stream) {
+                                       int page_size, int window, float scale, int rows, hipStream_t stream) {
+  PYLON_REQUIRE(rows == 64 || rows == 128, "attention_prefill: 64 or 128 query rows per workgroup, got %d", rows);
   PYLON_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "attention_prefill: %d query heads cannot be grouped over %d key/value heads", n_heads,
                 n_kv_heads);
-  PYLON_REQUIRE(n_heads / n_kv_heads <= AP_ROWS, "attention_prefill: at most %d query heads per key/value head",
-                AP_ROWS);
+  PYLON_REQUIRE(n_heads / n_kv_heads <= rows, "attention_prefill: at most %d query heads per key/value head",
+                rows);
   PYLON_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256,
                 "attention_prefill: head_dim %d is not 64, 128 or 256", head_dim);
   PYLON_REQUIRE(page_size > 0 && table_width > 0 && window >= 0, "attention_prefill: bad page size, width or window");
+  PYLON_REQUIRE(table_width <= AP_TABLE, "attention_prefill: a request may hold at most %d pages, the table has %d columns",
+                AP_TABLE, table_width);
   PYLON_REQUIRE(n_kv_heads <= 65535, "attention_prefill: too many key/value heads for one launch");
   if (n_tiles == 0) return 0;
   const int group = n_heads / n_kv_heads;
   dim3 grid(n_tiles, n_kv_heads), block(256);
-#define GO(HD)                                                                                         \
-  hipLaunchKernelGGL((attention_prefill_kernel<HD>), grid, block, 0, stream, (uint16_t*)out,           \
-                     (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache,           \
-                     block_table, table_width, tiles, n_heads, n_kv_heads, group, page_size, window, scale)
-  if (head_dim == 64)
-    GO(64);
-  else if (head_dim == 128)
-    GO(128);
-  else
-    GO(256);
+  const bool pow2 = (page_size & (page_size - 1)) == 0;
+#define GO(HD, QT)                                                                                       \
+  do {                                                                                                   \
+    if (pow2)                                                                                            \
+      hipLaunchKernelGGL((attention_prefill_kernel<HD, QT, true>), grid, block, 0, stream, (uint16_t*)out, \
+                         (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache,         \
+                         block_table, table_width, tiles, n_heads, n_kv_heads, group, page_size, window, scale); \
+    else                                                                                                 \
+      hipLaunchKernelGGL((attention_prefill_kernel<HD, QT, false>), grid, block, 0, stream, (uint16_t*)out, \
+                         (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache,         \
+                         block_table, table_width, tiles, n_heads, n_kv_heads, group, page_size, window, scale); \
+  } while (0)
+  if (rows == 64) {
+    if (head_dim == 64) GO(64, 1);
+    else if (head_dim == 128) GO(128, 1);
+    else GO(256, 1);
+  } else {
+    if (head_dim == 64) GO(64, 2);
+    else if (head_dim == 128) GO(128, 2);
+    else GO(256, 2);
+  }
 #undef GO
   PYLON_LAUNCHED("attention_prefill");
 }

@@ -317,23 +317,36 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
     return out
 
 
-PREFILL_ROWS = 64  # (token, head) query rows one workgroup of the prefill kernel takes
+PREFILL_ROWS = 128  # most (token, head) query rows one workgroup of the prefill kernel takes
 
 
-def prefill_attention_ok(q: torch.Tensor, k_cache: torch.Tensor) -> bool:
+def prefill_rows(tokens: int, n_heads: int, group: int) -> int:
+    """Query rows per workgroup: 128 halve the traffic from LDS per matrix instruction, but a
+    step with few query rows fills more of the chip with workgroups of 64 (which hold a
+    group of at most 64 heads)."""
+    return 128 if tokens * n_heads >= 128 * 512 or group > 64 else 64
+
+
+PREFILL_MAX_PAGES = 4096  # block-table columns the prefill kernel keeps in LDS
+
+
+def prefill_attention_ok(q: torch.Tensor, k_cache: torch.Tensor, block_table: Optional[torch.Tensor] = None) -> bool:
     tokens, n_heads, head_dim = q.shape
     n_kv_heads = k_cache.shape[2]
     return (q.dtype == torch.bfloat16 and head_dim in DECODE_HEAD_DIMS and n_heads % n_kv_heads == 0
-            and n_heads // n_kv_heads <= PREFILL_ROWS)
+            and n_heads // n_kv_heads <= PREFILL_ROWS
+            and (block_table is None or block_table.shape[1] <= PREFILL_MAX_PAGES))
 
 
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_table: torch.Tensor, tiles: torch.Tensor, *, page_size: int,
-                      window: Optional[int], scale: float) -> torch.Tensor:
+                      window: Optional[int], scale: float, rows: Optional[int] = None) -> torch.Tensor:
     """Paged causal attention of bfloat16 prompt portions on the matrix cores.  ``tiles`` is
     int32 ``[n, 4]``: first token index, token count, block-table row and first position of
-    runs of at most ``128 // group`` consecutive tokens of one request."""
-    if q.dim() != 3 or not prefill_attention_ok(q, k_cache):
+    runs of at most ``rows // group`` consecutive tokens of one request; ``rows`` (64 or 128,
+    default :data:`PREFILL_ROWS`) is the number of query rows a workgroup takes."""
+    rows = rows or PREFILL_ROWS
+    if q.dim() != 3 or not prefill_attention_ok(q, k_cache, block_table):
         raise KernelError("attention_prefill does not take this geometry")
     tokens, n_heads, head_dim = q.shape
     pages, psize, n_kv_heads, hd = k_cache.shape
@@ -349,7 +362,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _lib.call("pylon_attention_prefill", _dev(out, "out"), _dev(q, "q"), _dev(k_cache, "k_cache"),
               _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
               _dev(tiles, "tiles", torch.int32), tiles.shape[0], n_heads, n_kv_heads, head_dim, page_size,
-              int(window or 0), float(scale), _stream())
+              int(window or 0), float(scale), int(rows), _stream())
     return out
 
 

@@ -80,11 +80,13 @@ class Attention(Part):
                 q, cache.k, cache.v, cache.block_table, None, ctx.positions,
                 page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits,
             )
-        elif ops.prefill_attention_ok(q, cache.k):
-            tiles = ctx.token_tiles(ops.PREFILL_ROWS // (spec.n_heads // spec.n_kv_heads))
+        elif ops.prefill_attention_ok(q, cache.k, cache.block_table):
+            group = spec.n_heads // spec.n_kv_heads
+            rows = ops.prefill_rows(tokens, spec.n_heads, group)
+            tiles = ctx.token_tiles(rows // group)
             context = ops.attention_prefill(
                 q, cache.k, cache.v, cache.block_table, tiles,
-                page_size=cache.page_size, window=spec.window, scale=spec.scale,
+                page_size=cache.page_size, window=spec.window, scale=spec.scale, rows=rows,
             )
         else:
             context = ops.paged_attention(

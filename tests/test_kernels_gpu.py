@@ -353,8 +353,10 @@ def test_attention_decode(ops, geom, n_splits):
 
 
 @pytest.mark.parametrize("geom", [(8, 2, 128, 64, None), (4, 4, 64, 16, None), (12, 2, 128, 32, 100),
-                                  (5, 1, 256, 16, None), (3, 3, 64, 256, 37), (16, 1, 128, 64, None)])
-def test_attention_prefill(ops, geom):
+                                  (5, 1, 256, 16, None), (3, 3, 64, 256, 37), (16, 1, 128, 64, None),
+                                  (8, 4, 128, 48, None), (6, 2, 64, 80, 90)])
+@pytest.mark.parametrize("rows", [64, 128])
+def test_attention_prefill(ops, geom, rows):
     """Portions of several requests at once: starting inside a page, a one-token portion, a
     portion with earlier context; pages in scrambled order, everything unheld poisoned."""
     nh, nkv, hd, page, window = geom
@@ -381,7 +383,7 @@ def test_attention_prefill(ops, geom):
                 kc[pg, off] = float("nan")
                 vc[pg, off] = float("nan")
     tok_row, positions, tiles = [], [], []
-    per_tile = ops.PREFILL_ROWS // group
+    per_tile = rows // group
     for r, (before, count) in enumerate(portions):
         for lo in range(0, count, per_tile):
             tiles.append((len(tok_row) + lo, min(per_tile, count - lo), r, before + lo))
@@ -392,7 +394,7 @@ def test_attention_prefill(ops, geom):
     scale = 1 / math.sqrt(hd)
     got = ops.attention_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV),
                                 torch.tensor(tiles, dtype=torch.int32, device=DEV),
-                                page_size=page, window=window, scale=scale)
+                                page_size=page, window=window, scale=scale, rows=rows)
     assert not torch.isnan(got.float()).any()
     kf, vf = f64(kc), f64(vc)
     worst = 0.0
