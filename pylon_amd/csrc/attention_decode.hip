@@ -9,6 +9,11 @@
 // meet in LDS and are merged in the order of the ranges, so no partial result ever goes
 // through global memory and there is no second kernel.
 //
+// Few tokens with long contexts would leave most of the chip idle that way.  Then the keys
+// of a (token, head) are first cut over several workgroups (gridDim.z); each leaves its
+// merged partial result (maximum, sum, unnormalised values, float) in a scratch buffer,
+// and a second small kernel merges those in the order of the cuts.
+//
 // Scores come from the 16x16x32 bf16 matrix instruction with 16 keys as rows and the
 // group's query heads as columns (unused columns are zero).  The weighted sum of values
 // runs on the vector units: a value row is read by head_dim/8 lanes, 16 bytes each, so one
@@ -66,7 +71,7 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, typename DecodeCache<PREP>::ptr k_cache,
     typename DecodeCache<PREP>::ptr v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tok_row, const int* __restrict__ positions, int n_heads, int n_kv_heads,
-    int page_size, int window, float scale, DecodePrep prep) {
+    int page_size, int window, float scale, DecodePrep prep, float* __restrict__ partial) {
   constexpr int HD = EPL * 64;
   constexpr int TILES = AD_SUPER / AD_TILE;
   // per wave: probabilities of the keys in flight; then the waves' partial results
@@ -88,14 +93,20 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
   const int table_entry = (lane < table_width) ? table[lane] : 0;
   const int pos = positions[t];
 
-  // the keys of this wave
+  // the keys of this workgroup (all of them unless gridDim.z cuts them), then of this wave
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int n_keys = pos + 1 - first;
+  const int n_cuts = gridDim.z, cut = blockIdx.z;
+  int per_cut = (pos + 1 - first + n_cuts - 1) / n_cuts;
+  per_cut = (per_cut + AD_TILE - 1) / AD_TILE * AD_TILE;
+  const int c_begin = first + cut * per_cut;
+  const int c_end = c_begin + per_cut < pos + 1 ? c_begin + per_cut : pos + 1;
+  const bool holds_last = pos >= c_begin && pos < c_begin + per_cut;  // true for exactly one cut
+  const int n_keys = c_end > c_begin ? c_end - c_begin : 0;
   int per_wave = (n_keys + n_waves - 1) / n_waves;
   per_wave = (per_wave + AD_TILE - 1) / AD_TILE * AD_TILE;
-  const int k_begin = first + wave * per_wave;
+  const int k_begin = c_begin + wave * per_wave;
   int k_end = k_begin + per_wave;
-  if (k_end > pos + 1) k_end = pos + 1;
+  if (k_end > c_end) k_end = c_end;
 
   if constexpr (PREP) {
     // 512/head_dim heads per wave at a time: the group's query heads into LDS, then this
@@ -104,7 +115,8 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
     // the token's rotation table, one private copy per wave: no workgroup barrier before use
     float* cs = reinterpret_cast<float*>(q_lds + GP * HD) + wave * HD;
     const uint16_t* row = prep.qkv + static_cast<size_t>(t) * prep.row_stride;
-    const int slot = prep.slot_map != nullptr ? prep.slot_map[t] : -1;
+    // the new key and value are stored by the one workgroup whose keys include them
+    const int slot = (prep.slot_map != nullptr && holds_last) ? prep.slot_map[t] : -1;
     const int jobs = group + (slot >= 0 ? 2 : 0);
     const int j = lane % LPH;
     // job -> where its head lies in the projection's row
@@ -298,11 +310,49 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
 #pragma unroll
       for (int i = 0; i < EPL; ++i) o[i] = fmaf(arow[lane * EPL + i], f, o[i]);
     }
-    const float inv = 1.0f / l;
-    uint16_t* orow = out + (static_cast<size_t>(t) * n_heads + kvh * group + h) * HD + lane * EPL;
+    if (n_cuts > 1) {
+      // [token][head][cut][HD values, maximum, sum]
+      float* prow = partial + ((static_cast<size_t>(t) * n_heads + kvh * group + h) * n_cuts + cut) * (HD + 2);
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) orow[i] = float_to_bf16_bits(o[i] * inv);
+      for (int i = 0; i < EPL; ++i) prow[lane * EPL + i] = o[i];
+      if (lane == 0) {
+        prow[HD] = m;
+        prow[HD + 1] = l;
+      }
+    } else {
+      const float inv = 1.0f / l;
+      uint16_t* orow = out + (static_cast<size_t>(t) * n_heads + kvh * group + h) * HD + lane * EPL;
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) orow[i] = float_to_bf16_bits(o[i] * inv);
+    }
   }
+}
+
+// One wave per (token, query head) merges the partial results of the cuts, in their order.
+template <int EPL>
+__global__ __launch_bounds__(PYLON_WAVE) void attention_decode_merge_kernel(
+    uint16_t* __restrict__ out, const float* __restrict__ partial, int n_heads, int n_cuts) {
+  constexpr int HD = EPL * 64;
+  const int lane = threadIdx.x;
+  const size_t row = static_cast<size_t>(blockIdx.y) * n_heads + blockIdx.x;
+  const float* prow = partial + row * n_cuts * (HD + 2);
+  float m = -INFINITY;
+  for (int c = 0; c < n_cuts; ++c) m = fmaxf(m, prow[c * (HD + 2) + HD]);
+  float l = 0.f, o[EPL];
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) o[i] = 0.f;
+  for (int c = 0; c < n_cuts; ++c) {
+    const float* pc = prow + c * (HD + 2);
+    const float lc = pc[HD + 1];
+    const float f = (lc == 0.f) ? 0.f : expf(pc[HD] - m);  // a cut without keys
+    l += lc * f;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) o[i] = fmaf(pc[lane * EPL + i], f, o[i]);
+  }
+  const float inv = 1.0f / l;
+  uint16_t* orow = out + row * HD + lane * EPL;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) orow[i] = float_to_bf16_bits(o[i] * inv);
 }
 
 static size_t decode_lds_bytes(int n_waves, int gp, int head_dim, bool prep) {
@@ -314,18 +364,19 @@ template <int EPL, bool PREP>
 static int launch_decode(void* out, const void* q, void* k_cache, void* v_cache,
                          const int* block_table, int table_width, const int* tok_row,
                          const int* positions, int tokens, int n_heads, int n_kv_heads, int page_size,
-                         int window, float scale, int n_waves, DecodePrep prep, hipStream_t stream) {
+                         int window, float scale, int n_waves, DecodePrep prep, int n_cuts, float* partial,
+                         hipStream_t stream) {
   const int group = n_heads / n_kv_heads;
   const int gp = group <= 1 ? 1 : group <= 2 ? 2 : group <= 4 ? 4 : group <= 8 ? 8 : 16;
   // the partial results of all waves have to fit into 64 KB of LDS
   while (n_waves > 1 && decode_lds_bytes(n_waves, gp, EPL * 64, PREP) > 65536) n_waves /= 2;
   const size_t lds = decode_lds_bytes(n_waves, gp, EPL * 64, PREP);
-  dim3 grid(n_kv_heads, tokens), block(n_waves * PYLON_WAVE);
+  dim3 grid(n_kv_heads, tokens, n_cuts), block(n_waves * PYLON_WAVE);
 #define LAUNCH(GP)                                                                                         \
   hipLaunchKernelGGL((attention_decode_kernel<EPL, EPL * 2, GP, PREP>), grid, block, lds, stream,          \
                      (uint16_t*)out, (const uint16_t*)q, (typename DecodeCache<PREP>::ptr)k_cache,         \
                      (typename DecodeCache<PREP>::ptr)v_cache, block_table, table_width, tok_row, positions, \
-                     n_heads, n_kv_heads, page_size, window, scale, prep)
+                     n_heads, n_kv_heads, page_size, window, scale, prep, partial)
   switch (gp) {
     case 1: LAUNCH(1); break;
     case 2: LAUNCH(2); break;
@@ -334,6 +385,25 @@ static int launch_decode(void* out, const void* q, void* k_cache, void* v_cache,
     default: LAUNCH(16); break;
   }
 #undef LAUNCH
+  if (n_cuts > 1)
+    hipLaunchKernelGGL((attention_decode_merge_kernel<EPL>), dim3(n_heads, tokens), dim3(PYLON_WAVE), 0, stream,
+                       (uint16_t*)out, partial, n_heads, n_cuts);
+  return 0;
+}
+
+// Floats of scratch that n_cuts > 1 needs.
+extern "C" long long pylon_attention_decode_scratch_floats(int tokens, int n_heads, int head_dim, int n_cuts) {
+  if (n_cuts <= 1) return 0;
+  return static_cast<long long>(tokens) * n_heads * n_cuts * (head_dim + 2);
+}
+
+static int check_decode_cuts(const char* name, int tokens, int n_heads, int head_dim, int n_cuts,
+                             const float* partial, long long partial_floats) {
+  PYLON_REQUIRE(n_cuts >= 1 && n_cuts <= 64, "%s: the keys can be cut over 1..64 workgroups, got %d", name, n_cuts);
+  PYLON_REQUIRE(n_cuts == 1 || (partial != nullptr && partial_floats >= pylon_attention_decode_scratch_floats(
+                                                                            tokens, n_heads, head_dim, n_cuts)),
+                "%s: %d cuts need a scratch buffer of %lld floats", name, n_cuts,
+                pylon_attention_decode_scratch_floats(tokens, n_heads, head_dim, n_cuts));
   return 0;
 }
 
@@ -353,21 +423,24 @@ static int check_decode_geometry(const char* name, int tokens, int n_heads, int 
 }
 
 // q, out: [tokens, n_heads, head_dim] bf16; n_waves (1, 2, 4 or 8) wavefronts share
-// the keys of one (token, key/value head).
+// the keys of one (token, key/value head), after n_cuts workgroups have shared them first
+// (n_cuts > 1 needs `partial`, scratch of pylon_attention_decode_scratch_floats floats).
 extern "C" int pylon_attention_decode(void* out, const void* q, const void* k_cache, const void* v_cache,
                                       const int* block_table, int table_width, const int* tok_row,
                                       const int* positions, int tokens, int n_heads, int n_kv_heads,
                                       int head_dim, int page_size, int window, float scale, int n_waves,
+                                      int n_cuts, float* partial, long long partial_floats,
                                       hipStream_t stream) {
   if (check_decode_geometry("attention_decode", tokens, n_heads, n_kv_heads, head_dim, page_size, table_width,
-                            window, n_waves))
+                            window, n_waves) ||
+      check_decode_cuts("attention_decode", tokens, n_heads, head_dim, n_cuts, partial, partial_floats))
     return 1;
   if (tokens == 0) return 0;
   const DecodePrep none = {};
 #define GO(D)                                                                                       \
   launch_decode<D, false>(out, q, const_cast<void*>(k_cache), const_cast<void*>(v_cache), block_table, \
                           table_width, tok_row, positions, tokens, n_heads, n_kv_heads, page_size, window, \
-                          scale, n_waves, none, stream)
+                          scale, n_waves, none, n_cuts, partial, stream)
   switch (head_dim / 64) {
     case 1: GO(1); break;
     case 2: GO(2); break;
@@ -388,9 +461,11 @@ extern "C" int pylon_attention_decode_fused(void* out, const void* qkv, long lon
                                             const int* slot_map, const int* block_table, int table_width,
                                             const int* tok_row, const int* positions, int tokens,
                                             int n_heads, int n_kv_heads, int head_dim, int page_size,
-                                            int window, float scale, int n_waves, hipStream_t stream) {
+                                            int window, float scale, int n_waves, int n_cuts,
+                                            float* partial, long long partial_floats, hipStream_t stream) {
   if (check_decode_geometry("attention_decode_fused", tokens, n_heads, n_kv_heads, head_dim, page_size,
-                            table_width, window, n_waves))
+                            table_width, window, n_waves) ||
+      check_decode_cuts("attention_decode_fused", tokens, n_heads, head_dim, n_cuts, partial, partial_floats))
     return 1;
   const long long heads = n_heads + (slot_map != nullptr ? 2ll * n_kv_heads : 0);
   PYLON_REQUIRE(row_stride >= heads * head_dim, "attention_decode_fused: row stride %lld is shorter than %lld heads of %d",
@@ -401,7 +476,7 @@ extern "C" int pylon_attention_decode_fused(void* out, const void* qkv, long lon
   const DecodePrep prep = {static_cast<const uint16_t*>(qkv), row_stride, q_weight, k_weight, eps, inv_freq, slot_map};
 #define GO(D)                                                                                            \
   launch_decode<D, true>(out, nullptr, k_cache, v_cache, block_table, table_width, tok_row, positions, tokens, \
-                         n_heads, n_kv_heads, page_size, window, scale, n_waves, prep, stream)
+                         n_heads, n_kv_heads, page_size, window, scale, n_waves, prep, n_cuts, partial, stream)
   switch (head_dim / 64) {
     case 1: GO(1); break;
     case 2: GO(2); break;

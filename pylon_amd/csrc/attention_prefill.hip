@@ -37,7 +37,7 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 // is a power of two, so a key's page and offset are a shift and a mask (a division by a
 // run-time number costs some twenty instructions, eight times per thread and block).
 template <int HD, int QT, bool POW2>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) void attention_prefill_kernel(
+__global__ __launch_bounds__(256) void attention_prefill_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, int n_heads, int n_kv_heads, int group, int page_size, int window,

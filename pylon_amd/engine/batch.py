@@ -101,7 +101,7 @@ class StepContext:
     counts: np.ndarray = field(default=None)
     starts: np.ndarray = field(default=None)
     max_count: int = 0
-    max_len: int = 0
+    max_len: int = 0  # the longest row after this step; with fixed_shapes an upper bound on it
     decode_only: bool = False
     fixed_shapes: bool = False  # launches must not depend on lengths (graph capture)
     logit_slots: Optional[torch.Tensor] = None  # int32 [n]: state slot of each wanted row's request
@@ -162,12 +162,13 @@ def plan_layout(tokens: int, rows: int, n_logits: int, n_groups: int, width: int
 def build_step(entries: Seq[StepEntry], manager: CacheManager, arena: MetadataArena, *,
                vocab_size: int, width: Optional[int] = None,
                device_block: Optional[torch.Tensor] = None, fixed_shapes: bool = False,
-               chosen: Optional[torch.Tensor] = None) -> StepContext:
+               chosen: Optional[torch.Tensor] = None, len_bound: Optional[int] = None) -> StepContext:
     """Check the entries, take the pages they need, and put the step's metadata on the
     device.  Raises before touching the cache if any entry is malformed; raises
     :class:`~pylon_amd.cache.pages.OutOfPages` (cache untouched) if pages run short.
     ``chosen`` is the table of last sampled tokens by state slot; only with it may an
-    entry hold :data:`PENDING`."""
+    entry hold :data:`PENDING`.  ``len_bound``: what the parts are told instead of the
+    longest row's length (a recorded step must not depend on the lengths themselves)."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     rows = len(entries)
@@ -249,6 +250,7 @@ def build_step(entries: Seq[StepEntry], manager: CacheManager, arena: MetadataAr
         logit_idx=dev("logit_idx") if logit_list else None, n_logits=len(logit_list),
         logit_slots=dev("logit_slots") if logit_list else None, chosen=chosen,
         views=views, counts=counts, starts=starts, max_count=int(counts.max()),
-        max_len=int(seq_lens.max()), decode_only=bool((counts == 1).all()),
+        max_len=int(seq_lens.max()) if len_bound is None else int(len_bound),
+        decode_only=bool((counts == 1).all()),
         fixed_shapes=fixed_shapes,
     )

@@ -9,8 +9,10 @@ the first time a batch size is seen rather than all at start-up, and a batch is 
 padded to a larger captured size.
 
 The launches recorded in a graph must not depend on the requests' lengths: the block
-table has a fixed width, and the decode attention kernel cuts keys into a number of
-ranges that depends on the batch size only.
+table has a fixed width, and how the decode attention kernel shares a request's keys
+between workgroups and waves depends on the batch size and on a bound on the lengths
+only.  That bound is a power of two of at least 1024 tokens; there is one graph per
+(batch size, bound).
 """
 from __future__ import annotations
 
@@ -39,17 +41,25 @@ class DecodeGraphs:
         self.max_batch = max_batch
         self.width = max_pages_per_request
         self.pool = torch.cuda.graph_pool_handle()
-        self.captured: Dict[int, tuple] = {}
+        self.captured: Dict[Tuple[int, int], tuple] = {}
         self.failed = set()
         self.replays = 0
 
     def captured_sizes(self):
-        return tuple(sorted(self.captured))
+        return tuple(sorted({rows for rows, _bound in self.captured}))
+
+    def _bound(self, entries: Seq[StepEntry]) -> int:
+        """The power of two (from 1024) that holds the longest request after this step."""
+        need = max(e.seq.length for e in entries) + 1
+        bound = 1024
+        while bound < need:
+            bound *= 2
+        return bound
 
     def wants(self, entries: Seq[StepEntry]) -> bool:
         """A decode-only step: one token per request, each wanting its logits."""
         rows = len(entries)
-        if rows > self.max_batch or rows in self.failed:
+        if rows > self.max_batch or (rows, self._bound(entries)) in self.failed:
             return False
         page = self.manager.page_size
         for e in entries:
@@ -66,13 +76,15 @@ class DecodeGraphs:
         rows = len(entries)
         manager, model, arena = self.manager, self.model, self.arena
         pairs = [(e.seq, 1) for e in entries]
-        entry = self.captured.get(rows)
+        bound = self._bound(entries)
+        key = (rows, bound)
+        entry = self.captured.get(key)
         if entry is None:
             _, size = plan_layout(rows, rows, rows, len(manager.groups), self.width)
             block = torch.empty(size, dtype=torch.int32, device=model.device)
             ctx = build_step(entries, manager, arena, vocab_size=model.spec.vocab_size,
                              width=self.width, device_block=block, fixed_shapes=True,
-                             chosen=self.chosen)
+                             chosen=self.chosen, len_bound=bound)
             # No garbage collection while the stream is capturing: a finalizer that frees a
             # device object (an event, another graph) is not allowed there and aborts.
             gc.collect()
@@ -84,20 +96,21 @@ class DecodeGraphs:
                 with torch.cuda.graph(graph, pool=self.pool):
                     logits = model.step(ctx)
             except Exception:  # noqa: BLE001 - a failed capture leaves this size to eager steps
-                logger.exception("decode_graph_capture_failed batch_size=%s", rows)
-                self.failed.add(rows)
+                logger.exception("decode_graph_capture_failed batch_size=%s bound=%s", rows, bound)
+                self.failed.add(key)
                 manager.cancel(pairs)
                 return None
             finally:
                 if gc_was_enabled:
                     gc.enable()
-            self.captured[rows] = (graph, block, logits, ctx.logit_slots)
+            self.captured[key] = (graph, block, logits, ctx.logit_slots)
             self.last_logit_slots = ctx.logit_slots
             graph.replay()  # capture records only; this runs the step
         else:
             graph, block, logits, self.last_logit_slots = entry
             build_step(entries, manager, arena, vocab_size=model.spec.vocab_size,
-                       width=self.width, device_block=block, fixed_shapes=True, chosen=self.chosen)
+                       width=self.width, device_block=block, fixed_shapes=True, chosen=self.chosen,
+                       len_bound=bound)
             graph.replay()
         self.replays += 1
         manager.commit(pairs)

@@ -232,13 +232,36 @@ def decode_splits(tokens: int, n_kv_heads: int, max_len: Optional[int]) -> int:
     return waves
 
 
+def decode_cuts(tokens: int, n_kv_heads: int, max_len: Optional[int]) -> int:
+    """Workgroups that share the keys of one (token, key/value head) before the waves of
+    each share theirs: more than one when a few long requests would otherwise occupy a
+    fraction of the chip.  Measured on 256 compute units: about 256 workgroups in all, each
+    with at least 1024 keys of ``max_len`` (which may be an upper bound well above the true
+    lengths).  E.g. 8 tokens of 8192 keys: 53 us with 4 cuts, 102 us with one; more cuts
+    than that lose again to the second kernel and its partial results."""
+    cuts = 1
+    if max_len is None:
+        return cuts
+    while tokens * n_kv_heads * cuts * 2 <= 256 and max_len // (cuts * 2) >= 1024 and cuts < 64:
+        cuts *= 2
+    return cuts
+
+
+def _decode_scratch(tokens: int, n_heads: int, head_dim: int, n_cuts: int, device) -> Optional[torch.Tensor]:
+    if n_cuts <= 1:
+        return None
+    return torch.empty((tokens * n_heads * n_cuts * (head_dim + 2),), dtype=torch.float32, device=device)
+
+
 def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                      block_table: torch.Tensor, tok_row: Optional[torch.Tensor], positions: torch.Tensor, *,
-                     page_size: int, window: Optional[int], scale: float, n_splits: int) -> torch.Tensor:
+                     page_size: int, window: Optional[int], scale: float, n_splits: int,
+                     n_cuts: int = 1) -> torch.Tensor:
     """Paged attention of a few bfloat16 query tokens; ``n_splits`` wavefronts share the
-    keys of each (token, key/value head) and merge their partial results.  ``tok_row`` None
-    means token ``t`` uses row ``t`` of the block table (a decode-only step), which saves
-    the kernel one dependent trip to memory."""
+    keys of each (token, key/value head) and merge their partial results, after ``n_cuts``
+    workgroups have shared them first (their partial results meet in a second small
+    kernel).  ``tok_row`` None means token ``t`` uses row ``t`` of the block table (a
+    decode-only step), which saves the kernel one dependent trip to memory."""
     if q.dim() != 3 or not decode_attention_ok(q, k_cache):
         raise KernelError("attention_decode does not take this geometry")
     tokens, n_heads, head_dim = q.shape
@@ -257,11 +280,13 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     elif tok_row.numel() != tokens:
         raise KernelError("attention_decode: one row id per token is required")
     out = torch.empty_like(q)
+    scratch = _decode_scratch(tokens, n_heads, head_dim, n_cuts, q.device)
     _lib.call("pylon_attention_decode", _dev(out, "out"), _dev(q, "q"), _dev(k_cache, "k_cache"),
               _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
               _dev(tok_row, "tok_row", torch.int32), _dev(positions, "positions", torch.int32),
               tokens, n_heads, n_kv_heads, head_dim, page_size, int(window or 0), float(scale),
-              int(n_splits), _stream())
+              int(n_splits), int(n_cuts), _dev(scratch, "scratch"), 0 if scratch is None else scratch.numel(),
+              _stream())
     return out
 
 
@@ -280,7 +305,8 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
                            block_table: torch.Tensor, tok_row: Optional[torch.Tensor], positions: torch.Tensor, *,
                            n_heads: int, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
                            eps: float, inv_freq: Optional[torch.Tensor], slot_map: Optional[torch.Tensor],
-                           page_size: int, window: Optional[int], scale: float, n_splits: int) -> torch.Tensor:
+                           page_size: int, window: Optional[int], scale: float, n_splits: int,
+                           n_cuts: int = 1) -> torch.Tensor:
     """:func:`qkv_prepare` and :func:`attention_decode` in one launch: from the raw projection
     ``qkv`` ``[tokens, (n_heads + 2 kv_heads) * head_dim]`` (``[tokens, n_heads * head_dim]``
     when ``slot_map`` is None and nothing is stored).  Returns ``[tokens, n_heads, head_dim]``."""
@@ -307,13 +333,15 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
     elif tok_row.numel() != tokens:
         raise KernelError("attention_decode_fused: one row id per token is required")
     out = torch.empty((tokens, n_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+    scratch = _decode_scratch(tokens, n_heads, head_dim, n_cuts, qkv.device)
     _lib.call("pylon_attention_decode_fused", _dev(out, "out"), qkv.data_ptr(), qkv.stride(0),
               _dev(q_weight, "q_weight", torch.float32), _dev(k_weight, "k_weight", torch.float32), float(eps),
               _dev(inv_freq, "inv_freq", torch.float32), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
               _dev(slot_map, "slot_map", torch.int32), _dev(block_table, "block_table", torch.int32),
               block_table.shape[1], _dev(tok_row, "tok_row", torch.int32),
               _dev(positions, "positions", torch.int32), tokens, n_heads, n_kv_heads, head_dim, page_size,
-              int(window or 0), float(scale), int(n_splits), _stream())
+              int(window or 0), float(scale), int(n_splits), int(n_cuts), _dev(scratch, "scratch"),
+              0 if scratch is None else scratch.numel(), _stream())
     return out
 
 

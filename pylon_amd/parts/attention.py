@@ -42,6 +42,10 @@ class Attention(Part):
     def cache_requirement(self) -> KVRequirement:
         return KVRequirement(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window)
 
+    def _span(self, ctx) -> int:
+        """The most keys a token of this step attends to."""
+        return ctx.max_len if self.spec.window is None else min(ctx.max_len, self.spec.window)
+
     def forward(self, h: torch.Tensor, ctx, cache, stores: bool) -> torch.Tensor:
         spec = self.spec
         tokens = h.shape[0]
@@ -54,13 +58,14 @@ class Attention(Part):
                 qkv, cache.k, tokens=tokens, n_heads=spec.n_heads, head_dim=spec.head_dim,
                 rot_dim=rotary[1] if rotary else 0):
             # one launch norms and rotates q and k, stores k and v, and attends
-            splits = ops.decode_splits(tokens, spec.n_kv_heads, None if ctx.fixed_shapes else ctx.max_len)
+            cuts = ops.decode_cuts(tokens, spec.n_kv_heads, self._span(ctx))
+            splits = ops.decode_splits(tokens * cuts, spec.n_kv_heads, -(-self._span(ctx) // cuts))
             context = ops.attention_decode_fused(
                 qkv, cache.k, cache.v, cache.block_table, None, ctx.positions,
                 n_heads=spec.n_heads, q_weight=self.params.get("q_norm"), k_weight=self.params.get("k_norm"),
                 eps=spec.qk_norm_eps, inv_freq=rotary[0] if rotary else None,
                 slot_map=cache.slot_map if stores else None,
-                page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits,
+                page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits, n_cuts=cuts,
             )
             return ops.linear_for_residual(context.view(tokens, spec.q_size), self.params["out"],
                                            out_dtype=self.dtype)
@@ -74,11 +79,12 @@ class Attention(Part):
             positions=ctx.positions, slot_map=cache.slot_map, store_kv=stores,
         )
         if ctx.decode_only and ops.decode_attention_ok(q, cache.k):
-            splits = ops.decode_splits(tokens, spec.n_kv_heads, None if ctx.fixed_shapes else ctx.max_len)
+            cuts = ops.decode_cuts(tokens, spec.n_kv_heads, self._span(ctx))
+            splits = ops.decode_splits(tokens * cuts, spec.n_kv_heads, -(-self._span(ctx) // cuts))
             # in a decode-only step token t is row t
             context = ops.attention_decode(
                 q, cache.k, cache.v, cache.block_table, None, ctx.positions,
-                page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits,
+                page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits, n_cuts=cuts,
             )
         elif ops.prefill_attention_ok(q, cache.k, cache.block_table):
             group = spec.n_heads // spec.n_kv_heads

@@ -41,10 +41,18 @@ TINY_C = _qwen3(
     intermediate_size=176, vocab_size=301, rope_theta=500000.0, rms_norm_eps=3e-6,
     tie_word_embeddings=False, max_position_embeddings=2048,
 )
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-# A has unit norm weights; B and C draw them, so that a kernel ignoring a norm weight fails.
-NORM_JITTER = {"A": 0.0, "B": 0.2, "C": 0.2}
-SEEDS = {"A": 11, "B": 23, "C": 37}
+# D has a head size that the matrix-core attention kernels take (A, B and C run on the
+# general kernel), three query heads per key/value head, and room for contexts long enough
+# that a request's keys are shared between workgroups.
+TINY_D = _qwen3(
+    num_hidden_layers=2, hidden_size=112, num_attention_heads=6, num_key_value_heads=2, head_dim=64,
+    intermediate_size=208, vocab_size=331, rope_theta=250000.0, rms_norm_eps=2e-6,
+    tie_word_embeddings=True, max_position_embeddings=4096,
+)
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+# A has unit norm weights; the others draw them, so that a kernel ignoring a norm weight fails.
+NORM_JITTER = {"A": 0.0, "B": 0.2, "C": 0.2, "D": 0.2}
+SEEDS = {"A": 11, "B": 23, "C": 37, "D": 41}
 
 
 def make_model_folder(tmp: Path, name: str, *, dtype: str = "float32", config=None, seed=None,

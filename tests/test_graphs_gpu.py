@@ -84,3 +84,46 @@ def test_a_request_longer_than_the_captured_table_runs_eagerly(tmp_path):
     for t in toks[28:40]:
         runner.step([StepEntry(seq, [t], [0])])
     assert runner.graphs.replays == 4 and seq.length == 40  # positions 28..31 fit the table
+
+
+def test_long_requests_share_their_keys_between_workgroups_in_graphs_too(tmp_path):
+    """Two requests around a thousand tokens, decoded while they cross the length bound
+    that a graph is recorded for: with and without graphs, the decode attention cuts their
+    keys over several workgroups, and both give the plain model's logits."""
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from pylon_amd.engine import Runner, StepEntry
+    from pylon_amd.kernels import ops
+
+    folder = make_model_folder(tmp_path, "D", dtype="bfloat16", std=0.08)
+    cfg, weights = read_folder(folder)
+    vocab = cfg["vocab_size"]
+    prompts = {"long": random_tokens(vocab, 2030, 1), "other": random_tokens(vocab, 700, 2)}
+    decode = {rid: random_tokens(vocab, 40, 10 + i) for i, rid in enumerate(prompts)}
+    assert ops.decode_cuts(2, cfg["num_key_value_heads"], 2048) > 1
+
+    def run(graphs):
+        runner = Runner.from_folder(folder, dtype="bfloat16", page_size=64, num_pages=48, max_requests=2)
+        if graphs:
+            runner.enable_graphs(2, max_tokens_per_request=4096)
+        seqs = {rid: runner.open(rid) for rid in prompts}
+        rows = {rid: [] for rid in prompts}
+        for rid, seq in seqs.items():
+            out = runner.step([StepEntry(seq, prompts[rid], [len(prompts[rid]) - 1])])
+            rows[rid].append(out[0].cpu().numpy())
+        for i in range(39):
+            out = runner.step([StepEntry(seqs[rid], [decode[rid][i]], [0]) for rid in prompts]).cpu().numpy()
+            for r, rid in enumerate(prompts):
+                rows[rid].append(out[r])
+        return runner, {rid: np.stack(r) for rid, r in rows.items()}
+
+    eager_runner, eager = run(False)
+    graph_runner, graphed = run(True)
+    assert {bound for _rows, bound in graph_runner.graphs.captured} == {2048, 4096}
+    for rid in prompts:
+        toks = prompts[rid] + decode[rid][:39]
+        want = plain.forward(weights, cfg, toks)[len(prompts[rid]) - 1:]
+        scale = np.abs(want).max()
+        assert np.abs(eager[rid] - want).max() <= 2e-2 * scale, rid
+        assert np.abs(graphed[rid] - want).max() <= 2e-2 * scale, rid
+        assert np.abs(graphed[rid] - eager[rid]).max() <= 1e-2 * scale, rid

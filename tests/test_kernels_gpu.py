@@ -300,8 +300,10 @@ def test_paged_attention(ops, dtype, geom):
 
 @pytest.mark.parametrize("geom", [(8, 2, 128, 64, None), (4, 4, 64, 16, None), (16, 1, 256, 32, 100),
                                   (6, 2, 128, 256, None), (1, 1, 64, 16, 7)])
-@pytest.mark.parametrize("n_splits", [1, 2, 4, 8])
-def test_attention_decode(ops, geom, n_splits):
+@pytest.mark.parametrize("n_splits,n_cuts", [(1, 1), (2, 1), (4, 1), (8, 1), (1, 2), (4, 3), (8, 8), (2, 64)])
+def test_attention_decode(ops, geom, n_splits, n_cuts):
+    """Keys shared between the waves of a workgroup (n_splits) and, before that, between
+    workgroups (n_cuts): also with more shares than a short request has keys."""
     nh, nkv, hd, page, window = geom
     dtype = torch.bfloat16
     lengths = [1, 15, 16, 17, 65, 300, 2 * page + 1, 700]
@@ -333,7 +335,9 @@ def test_attention_decode(ops, geom, n_splits):
     args = (q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV),
             torch.tensor(rows, dtype=torch.int32, device=DEV),
             torch.tensor(positions, dtype=torch.int32, device=DEV))
-    got = ops.attention_decode(*args, page_size=page, window=window, scale=scale, n_splits=n_splits)
+    got = ops.attention_decode(*args, page_size=page, window=window, scale=scale, n_splits=n_splits,
+                               n_cuts=n_cuts)
+    assert not torch.isnan(got.float()).any()
     kf, vf = f64(kc), f64(vc)
     for i, (r, p) in enumerate(zip(rows, positions)):
         idx = [(int(table[r, j // page]), j % page) for j in range(p + 1)]
@@ -348,7 +352,7 @@ def test_attention_decode(ops, geom, n_splits):
     # without row ids token t uses row t of the table
     permuted = table[rows].contiguous()
     same = ops.attention_decode(args[0], args[1], args[2], permuted.to(DEV), None, args[5],
-                                page_size=page, window=window, scale=scale, n_splits=n_splits)
+                                page_size=page, window=window, scale=scale, n_splits=n_splits, n_cuts=n_cuts)
     assert torch.equal(same, got)
 
 
@@ -635,18 +639,18 @@ def test_decode_attention_that_prepares_q_k_v_itself(ops, geom, store):
     vc = rnd((total_pages, page, nkv, hd), 55, torch.bfloat16).to(DEV)
     kc2, vc2 = kc.clone(), vc.clone()
     for window in (None, 50):
-        for splits in (1, 4, 8):
+        for splits, cuts in ((1, 1), (4, 1), (8, 1), (2, 3), (8, 4)):
             q = torch.empty((tokens, nh, hd), dtype=torch.bfloat16, device=DEV)
             ops.qkv_prepare(qkv, q, kc, vc, n_heads=nh, n_kv_heads=nkv, head_dim=hd, q_weight=qw, k_weight=kw,
                             eps=eps, inv_freq=inv_freq, rot_dim=hd if rotated else 0,
                             positions=positions.to(DEV), slot_map=slots.to(DEV), store_kv=store)
             want = ops.attention_decode(q, kc, vc, table.to(DEV), None, positions.to(DEV), page_size=page,
-                                        window=window, scale=hd ** -0.5, n_splits=splits)
+                                        window=window, scale=hd ** -0.5, n_splits=splits, n_cuts=cuts)
             got = ops.attention_decode_fused(
                 qkv, kc2, vc2, table.to(DEV), None, positions.to(DEV), n_heads=nh, q_weight=qw, k_weight=kw,
                 eps=eps, inv_freq=inv_freq, slot_map=slots.to(DEV) if store else None, page_size=page,
-                window=window, scale=hd ** -0.5, n_splits=splits)
-            assert torch.equal(got, want), (window, splits)
+                window=window, scale=hd ** -0.5, n_splits=splits, n_cuts=cuts)
+            assert torch.equal(got, want), (window, splits, cuts)
             assert torch.equal(kc2, kc) and torch.equal(vc2, vc)
 
 
