@@ -1,7 +1,9 @@
 // out[M, N] = x[M, K] * w[N, K]^T for a few rows of x (M <= 64) in bfloat16: the matrix
 // products of a decode step, which are bound by reading w from memory exactly once.
 //
-// A workgroup of 4 or 8 wavefronts owns 16 rows of w (16 output columns).  The waves take
+// A workgroup of 4 or 8 wavefronts owns 16 rows of w (16 output columns), or 32 rows as two
+// tiles for matrices with many rows (the rows of x it loads then serve both; measured
+// 151 us against 165 us for a 151936 x 2560 matrix).  The waves take
 // turns along K in steps of 64: in a step a wave reads one full 128-byte line of each of
 // its 16 rows, as two loads that each cover a contiguous 64-byte half of every line.
 // All loads of a batch of steps are issued before the first product, so a wave with few
@@ -38,16 +40,17 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
-template <int MT, int WAVES, bool GLU, typename TO>
+// RT: 16-row tiles of w per workgroup (with GLU: one tile of gate rows and one of up rows)
+template <int MT, int WAVES, bool GLU, int RT, typename TO>
 __global__ __launch_bounds__(WAVES* PYLON_WAVE) void gemm_skinny_kernel(
     TO* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int M, int N,
     int K, long long ldx, long long ldw, long long ldo, long long part_stride) {
-  constexpr int TILES = GLU ? 2 : 1;  // row tiles of w per workgroup
+  constexpr int TILES = GLU ? 2 : RT;  // row tiles of w per workgroup
   __shared__ floatx4 red[WAVES][TILES][MT][PYLON_WAVE];
   const int lane = threadIdx.x & (PYLON_WAVE - 1);
   const int wave = threadIdx.x / PYLON_WAVE;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * (GLU ? 1 : RT);
   const int parts = gridDim.y, part = blockIdx.y;
 
   const int steps = (K + SK_STEP - 1) / SK_STEP;
@@ -55,10 +58,13 @@ __global__ __launch_bounds__(WAVES* PYLON_WAVE) void gemm_skinny_kernel(
   const int s_begin = part * per_part;
   const int s_end = (s_begin + per_part < steps) ? s_begin + per_part : steps;
 
-  const int wrow = (n0 + r < N) ? n0 + r : N - 1;
   const uint16_t* wp[TILES];
-  wp[0] = w + static_cast<size_t>(wrow) * ldw;
-  if (GLU) wp[TILES - 1] = w + static_cast<size_t>(N + wrow) * ldw;
+#pragma unroll
+  for (int j = 0; j < TILES; ++j) {
+    const int row = GLU ? n0 + r : n0 + 16 * j + r;
+    const int wrow = (row < N) ? row : N - 1;
+    wp[j] = w + static_cast<size_t>((GLU && j == 1) ? N + wrow : wrow) * ldw;
+  }
   const uint16_t* xp[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -72,7 +78,7 @@ __global__ __launch_bounds__(WAVES* PYLON_WAVE) void gemm_skinny_kernel(
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[j][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  constexpr int BATCH = (MT == 1) ? (GLU ? 5 : 10) : (MT == 2 ? 4 : 2);
+  constexpr int BATCH = (MT == 1) ? (TILES == 2 ? 5 : 10) : (MT == 2 ? 4 : 2) / (TILES == 2 && !GLU ? 2 : 1);
   for (int s0 = s_begin + wave; s0 < s_end; s0 += WAVES * BATCH) {
     bf16x8 a[BATCH][TILES][2], b[BATCH][MT][2];
 #pragma unroll
@@ -120,28 +126,36 @@ __global__ __launch_bounds__(WAVES* PYLON_WAVE) void gemm_skinny_kernel(
     const int m = t * 16 + r;
     if (m < M) {
       TO* dst = out + static_cast<size_t>(part) * part_stride + static_cast<size_t>(m) * ldo;
+      if (GLU) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int n = n0 + 4 * g + i;
-        if (n < N) {
-          const float v = GLU ? silu_f(sum[0][i]) * sum[TILES - 1][i] : sum[0][i];
-          dst[n] = from_float<TO>(v);
+        for (int i = 0; i < 4; ++i) {
+          const int n = n0 + 4 * g + i;
+          if (n < N) dst[n] = from_float<TO>(silu_f(sum[0][i]) * sum[TILES - 1][i]);
         }
+      } else {
+#pragma unroll
+        for (int j = 0; j < TILES; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int n = n0 + 16 * j + 4 * g + i;
+            if (n < N) dst[n] = from_float<TO>(sum[j][i]);
+          }
       }
     }
   }
 }
 
-template <int MT, int WAVES, bool GLU>
+template <int MT, int WAVES, bool GLU, int RT>
 static void launch_skinny(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                           long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
                           hipStream_t stream) {
-  dim3 grid((N + 15) / 16, parts), block(WAVES * PYLON_WAVE);
+  constexpr int ROWS = 16 * (GLU ? 1 : RT);
+  dim3 grid((N + ROWS - 1) / ROWS, parts), block(WAVES * PYLON_WAVE);
   if (out_dtype == PYLON_F32)
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WAVES, GLU, float>), grid, block, 0, stream, (float*)out,
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WAVES, GLU, RT, float>), grid, block, 0, stream, (float*)out,
                        (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride);
   else
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WAVES, GLU, bf16_t>), grid, block, 0, stream, (bf16_t*)out,
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, WAVES, GLU, RT, bf16_t>), grid, block, 0, stream, (bf16_t*)out,
                        (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride);
 }
 
@@ -153,11 +167,15 @@ static void launch_skinny_mt(void* out, int out_dtype, const void* x, const void
   // eight-wave form is kept for very long K only.
   const int steps = (K + SK_STEP - 1) / SK_STEP / parts;
   const bool wide = steps >= 512;
-#define GO(W, G) launch_skinny<MT, W, G>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream)
+#define GO(W, G, R) launch_skinny<MT, W, G, R>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream)
   if (glu) {
-    if (wide) GO(8, true); else GO(4, true);
+    if (wide) GO(8, true, 1); else GO(4, true, 1);
+  } else if (MT == 1 && parts == 1 && N >= 4096) {
+    // Two tiles of w per workgroup pay for one tile of x rows.  Matrices with few rows
+    // (which also cut K) keep one tile: they need the workgroups more than the saving.
+    if (wide) GO(8, false, 2); else GO(4, false, 2);
   } else {
-    if (wide) GO(8, false); else GO(4, false);
+    if (wide) GO(8, false, 1); else GO(4, false, 1);
   }
 #undef GO
 }

@@ -468,10 +468,12 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype
 
 
 def k_parts(n: int, k: int) -> int:
-    """How many ranges to cut K into so that a matrix with few rows still fills the chip."""
+    """How many ranges to cut K into so that a matrix with few rows still fills the chip.
+    At most 4: the residual norm that adds the partial results loses more with 8 of them
+    (9.8 us against 6.5 us for 8 rows of 2560) than the product gains."""
     tiles = (n + 15) // 16
     parts = 1
-    while tiles * parts < 512 and parts < 8 and k // (parts * 2) >= 512:
+    while tiles * parts < 512 and parts < 4 and k // (parts * 2) >= 512:
         parts *= 2
     return parts
 
