@@ -163,6 +163,8 @@ def main() -> int:
     parser.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     parser.add_argument("--no-prefill", action="store_true")
+    parser.add_argument("--prefill-only", action="store_true",
+                        help="only the prefill measurement (for profiling); prints its part of the record")
     args = parser.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus must be 1")
@@ -179,6 +181,11 @@ def main() -> int:
                                num_pages=max_batch * pages_per_request, graphs=not args.no_graphs)
     dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
     steps = min(args.steps, CONTEXT_LENGTH - PROMPT_LEN - args.warmup)
+    if args.prefill_only:
+        seconds = prefill_run(runner, cfg, repeats=5, seed=2)
+        print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
+                                      "ms": round(1e3 * seconds, 3)}}))
+        return 0
 
     elapsed, mean_context = decode_run(runner, cfg, args.batch, steps, args.warmup, seed=1)
     ms_per_step = 1e3 * elapsed / steps
