@@ -25,7 +25,6 @@ from concurrent.futures import Future
 from dataclasses import dataclass, field
 from typing import Callable, Deque, Iterable, List, Optional, Sequence, Tuple
 
-from ..cache.pages import OutOfPages
 from ..config.engine_config import PylonConfig
 from ..sampling.params import Sampling
 from .batch import PENDING, StepEntry

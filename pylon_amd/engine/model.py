@@ -7,7 +7,7 @@ vocabulary head only at the tokens whose logits are wanted
 """
 from __future__ import annotations
 
-from typing import Dict, Iterator, List, Optional, Tuple
+from typing import List, Optional
 
 import torch
 

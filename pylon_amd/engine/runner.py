@@ -9,7 +9,7 @@ be replayed from a HIP graph.
 from __future__ import annotations
 
 from pathlib import Path
-from typing import Hashable, List, Optional, Sequence as Seq
+from typing import Hashable, Optional, Sequence as Seq
 
 import torch
 

@@ -1,5 +1,3 @@
-import json
-import os
 import sys
 from pathlib import Path
 

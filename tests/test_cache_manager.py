@@ -2,7 +2,6 @@
 step's metadata vectors."""
 import random
 
-import numpy as np
 import pytest
 import torch
 

@@ -1,12 +1,10 @@
 """Generation through the entry point against the plain implementation: greedy, seeded
 temperature sampling, the first tokens of a sequence, and long decoding."""
-from pathlib import Path
-
 import numpy as np
 import pytest
 import torch
 
-from tests.helpers import CONFIGS, make_model_folder, random_tokens, read_folder
+from tests.helpers import make_model_folder, random_tokens, read_folder
 from tests.plain import qwen3 as plain
 
 pytestmark = pytest.mark.gpu

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests.helpers import CONFIGS, make_model_folder, random_tokens, read_folder
+from tests.helpers import make_model_folder, random_tokens, read_folder
 from tests.plain import qwen3 as plain
 
 pytestmark = pytest.mark.gpu

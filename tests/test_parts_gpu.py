@@ -1,13 +1,12 @@
 """Each part of a layer alone against its plain formula, and a model whose layers differ
 (windows, a layer run twice, a run that borrows another run's cache)."""
 import dataclasses
-import math
 
 import numpy as np
 import pytest
 import torch
 
-from tests.helpers import CONFIGS, make_model_folder, random_tokens, read_folder
+from tests.helpers import make_model_folder, random_tokens, read_folder
 from tests.plain import qwen3 as plain
 
 pytestmark = pytest.mark.gpu
