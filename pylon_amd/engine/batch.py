@@ -106,19 +106,27 @@ class StepContext:
     fixed_shapes: bool = False  # launches must not depend on lengths (graph capture)
     logit_slots: Optional[torch.Tensor] = None  # int32 [n]: state slot of each wanted row's request
     chosen: Optional[torch.Tensor] = None  # int32 [slots]: last sampled token per state slot
-    _tiles: Dict[int, torch.Tensor] = field(default_factory=dict)
+    _tiles: Dict[Tuple[int, int], torch.Tensor] = field(default_factory=dict)
 
     def cache(self, cache_id: int) -> CacheView:
         return self.views[cache_id]
 
-    def token_tiles(self, tokens_per_tile: int) -> torch.Tensor:
-        """int32 ``[n, 4]`` on the device: the step's tokens cut into runs of at most
-        ``tokens_per_tile`` consecutive tokens of one row, as (index of the first token,
-        count, row, position of the first token), longest context first so that the
-        heaviest tiles start first."""
-        tiles = self._tiles.get(tokens_per_tile)
+    @property
+    def leading_singles(self) -> int:
+        """How many rows at the head of the step bring exactly one token (the decoding
+        requests, which the engine puts first): token t of them is row t."""
+        more = np.nonzero(self.counts != 1)[0]
+        return int(more[0]) if more.size else self.rows
+
+    def token_tiles(self, tokens_per_tile: int, skip_rows: int = 0) -> torch.Tensor:
+        """int32 ``[n, 4]`` on the device: the step's tokens (without those of the first
+        ``skip_rows`` rows) cut into runs of at most ``tokens_per_tile`` consecutive tokens
+        of one row, as (index of the first token, count, row, position of the first token),
+        longest context first so that the heaviest tiles start first."""
+        tiles = self._tiles.get((tokens_per_tile, skip_rows))
         if tiles is None:
             per_row = -(-self.counts // tokens_per_tile)
+            per_row[:skip_rows] = 0
             row = np.repeat(np.arange(self.rows, dtype=np.int64), per_row)
             first_of_row = np.zeros(self.rows + 1, dtype=np.int64)
             np.cumsum(per_row, out=first_of_row[1:])
@@ -130,7 +138,7 @@ class StepContext:
             order = np.argsort(-(table[:, 3] + table[:, 1]), kind="stable")
             host = torch.from_numpy(np.ascontiguousarray(table[order].astype(np.int32)))
             tiles = host.to(self.token_ids.device)
-            self._tiles[tokens_per_tile] = tiles
+            self._tiles[(tokens_per_tile, skip_rows)] = tiles
         return tiles
 
 

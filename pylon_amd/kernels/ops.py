@@ -232,6 +232,14 @@ def decode_splits(tokens: int, n_kv_heads: int, max_len: Optional[int]) -> int:
     return waves
 
 
+def _like(q: torch.Tensor, out: Optional[torch.Tensor], name: str) -> torch.Tensor:
+    if out is None:
+        return torch.empty_like(q)
+    if out.shape != q.shape or out.dtype != q.dtype or not out.is_contiguous():
+        raise KernelError(f"{name}: out must be contiguous and of q's shape and dtype")
+    return out
+
+
 def decode_cuts(tokens: int, n_kv_heads: int, max_len: Optional[int]) -> int:
     """Workgroups that share the keys of one (token, key/value head) before the waves of
     each share theirs: more than one when a few long requests would otherwise occupy a
@@ -256,7 +264,7 @@ def _decode_scratch(tokens: int, n_heads: int, head_dim: int, n_cuts: int, devic
 def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                      block_table: torch.Tensor, tok_row: Optional[torch.Tensor], positions: torch.Tensor, *,
                      page_size: int, window: Optional[int], scale: float, n_splits: int,
-                     n_cuts: int = 1) -> torch.Tensor:
+                     n_cuts: int = 1, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Paged attention of a few bfloat16 query tokens; ``n_splits`` wavefronts share the
     keys of each (token, key/value head) and merge their partial results, after ``n_cuts``
     workgroups have shared them first (their partial results meet in a second small
@@ -279,7 +287,7 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
             raise KernelError("attention_decode: without row ids the table needs a row per token")
     elif tok_row.numel() != tokens:
         raise KernelError("attention_decode: one row id per token is required")
-    out = torch.empty_like(q)
+    out = _like(q, out, "attention_decode")
     scratch = _decode_scratch(tokens, n_heads, head_dim, n_cuts, q.device)
     _lib.call("pylon_attention_decode", _dev(out, "out"), _dev(q, "q"), _dev(k_cache, "k_cache"),
               _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
@@ -368,7 +376,8 @@ def prefill_attention_ok(q: torch.Tensor, k_cache: torch.Tensor, block_table: Op
 
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_table: torch.Tensor, tiles: torch.Tensor, *, page_size: int,
-                      window: Optional[int], scale: float, rows: Optional[int] = None) -> torch.Tensor:
+                      window: Optional[int], scale: float, rows: Optional[int] = None,
+                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Paged causal attention of bfloat16 prompt portions on the matrix cores.  ``tiles`` is
     int32 ``[n, 4]``: first token index, token count, block-table row and first position of
     runs of at most ``rows // group`` consecutive tokens of one request; ``rows`` (64 or 128,
@@ -386,7 +395,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         raise KernelError("attention_prefill: the cache holds more slots than an int32 can index")
     if tiles.dim() != 2 or tiles.shape[1] != 4 or block_table.dim() != 2:
         raise KernelError("attention_prefill: tiles must be [n, 4] and the block table 2-D")
-    out = torch.empty_like(q)
+    out = _like(q, out, "attention_prefill")  # rows that no tile covers are left as they are
     _lib.call("pylon_attention_prefill", _dev(out, "out"), _dev(q, "q"), _dev(k_cache, "k_cache"),
               _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
               _dev(tiles, "tiles", torch.int32), tiles.shape[0], n_heads, n_kv_heads, head_dim, page_size,

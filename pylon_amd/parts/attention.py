@@ -89,11 +89,29 @@ class Attention(Part):
         elif ops.prefill_attention_ok(q, cache.k, cache.block_table):
             group = spec.n_heads // spec.n_kv_heads
             rows = ops.prefill_rows(tokens, spec.n_heads, group)
-            tiles = ctx.token_tiles(rows // group)
-            context = ops.attention_prefill(
-                q, cache.k, cache.v, cache.block_table, tiles,
-                page_size=cache.page_size, window=spec.window, scale=spec.scale, rows=rows,
-            )
+            context = torch.empty_like(q)
+            # Decoding requests at the head of a mixed step go to the decode kernel (a
+            # single query row would walk a long context alone in a prefill workgroup).
+            singles = ctx.leading_singles
+            if not (0 < singles <= ops.DECODE_MAX_TOKENS and ops.decode_attention_ok(q[:singles], cache.k)):
+                singles = 0
+            if singles:
+                span = int(ctx.starts[:singles].max()) + 1
+                if spec.window is not None:
+                    span = min(span, spec.window)
+                cuts = ops.decode_cuts(singles, spec.n_kv_heads, span)
+                splits = ops.decode_splits(singles * cuts, spec.n_kv_heads, -(-span // cuts))
+                ops.attention_decode(
+                    q[:singles], cache.k, cache.v, cache.block_table, None, ctx.positions[:singles],
+                    page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits,
+                    n_cuts=cuts, out=context[:singles],
+                )
+            if singles < ctx.rows:
+                tiles = ctx.token_tiles(rows // group, skip_rows=singles)
+                ops.attention_prefill(
+                    q, cache.k, cache.v, cache.block_table, tiles,
+                    page_size=cache.page_size, window=spec.window, scale=spec.scale, rows=rows, out=context,
+                )
         else:
             context = ops.paged_attention(
                 q, cache.k, cache.v, cache.block_table, ctx.tok_row, ctx.positions,
