@@ -4,7 +4,7 @@ The programming entry point works on token ids, as the reference's does
 (/root/reference/src/pylon/engine.py:241-253)::
 
     from pylon_amd import Engine, Sampling
-    engine = Engine.from_folder("model_dir", dtype="bfloat16")
+    engine = Engine.from_folder("model_dir", dtype="bfloat16")   # or Engine.from_random(config_dict, seed)
     future = engine.enqueue([1, 2, 3], eos_token_id=None, sampling=Sampling(max_new_tokens=16))
     engine.run_until_idle()
     print(future.result().output_ids)

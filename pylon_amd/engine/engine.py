@@ -174,6 +174,21 @@ class Engine:
         threaded = options.pop("threaded", False)
         return cls(PylonConfig(model_path=str(folder), **options), threaded=threaded)
 
+    @classmethod
+    def from_random(cls, model_config: dict, seed: int = 0, *, std: float = 0.02, norm_jitter: float = 0.0,
+                    **options) -> "Engine":
+        """An engine over random weights of the architecture and sizes that ``model_config``
+        (the contents of a config.json) names: the folder that the random-weights mode
+        writes from (config, seed), loaded like any other and then deleted."""
+        import tempfile
+
+        from ..weights import write_random_model
+
+        with tempfile.TemporaryDirectory(prefix="pylon_random_") as tmp:
+            folder = write_random_model(tmp, model_config, seed, dtype=options.get("dtype", "bfloat16"),
+                                        std=std, norm_jitter=norm_jitter)
+            return cls.from_folder(folder, **options)
+
     # ---- the public surface -------------------------------------------------------------
     def enqueue(self, input_ids: Sequence[int], eos_token_id=None, sampling: Optional[Sampling] = None,
                 request_id: Optional[str] = None) -> Future:

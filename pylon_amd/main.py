@@ -5,8 +5,10 @@ This engine has no server; the same knobs are options here (the environment vari
 still work as defaults), and the commands run on token ids:
 
     python main.py generate --model DIR --prompt-ids 1,2,3 [--prompt-ids ...]
+    python main.py generate --random config.json --seed 0 --prompt-ids 1,2,3
     python main.py random-model --config config.json --seed 0 --out DIR
     python main.py replay --model DIR --dtype float32 --out DIR --max-tokens N  < steps.jsonl
+    python main.py bench [bench.py's options]
 """
 from __future__ import annotations
 
@@ -30,6 +32,8 @@ def _add_serving_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--num-pages", type=int)
     p.add_argument("--cuda-graphs", action="store_true", default=None,
                    help="replay decode-only steps from HIP graphs")
+    p.add_argument("--no-run-ahead", dest="run_ahead", action="store_false", default=None,
+                   help="read every step's tokens before the next step is queued")
 
 
 def _parse_ids(text: str):
@@ -52,6 +56,7 @@ def _generate(args) -> int:
         batch_wait_ms=args.batch_wait_ms, max_gpu_utilization=args.max_gpu_utilization,
         kv_cache_headroom_ratio=args.kv_cache_headroom_ratio, admit_skip=args.admit_skip,
         page_size=args.page_size, num_pages=args.num_pages, cuda_graphs=args.cuda_graphs,
+        run_ahead=args.run_ahead,
     )
     prompts = [_parse_ids(text) for text in args.prompt_ids or []]
     if args.prompt_file:
@@ -61,7 +66,16 @@ def _generate(args) -> int:
         return 2
     sampling = Sampling(max_new_tokens=args.max_new_tokens, temperature=args.temperature,
                         top_p=args.top_p, seed=args.seed)
-    engine = Engine(config)
+    if args.random:
+        if args.model:
+            print("give --model or --random, not both", file=sys.stderr)
+            return 2
+        import dataclasses
+
+        options = {k: v for k, v in dataclasses.asdict(config).items() if k != "model_path"}
+        engine = Engine.from_random(json.loads(Path(args.random).read_text()), args.seed, **options)
+    else:
+        engine = Engine(config)
     try:
         eos = _parse_ids(args.eos_token_id) if args.eos_token_id else getattr(engine.runner.config, "eos_token_id", None)
         results = engine.generate(prompts, sampling, eos)
@@ -94,6 +108,8 @@ def main(argv=None) -> None:
 
     gen = sub.add_parser("generate", help="generate from prompts given as token ids")
     _add_serving_options(gen)
+    gen.add_argument("--random", metavar="CONFIG.json",
+                     help="instead of --model: random weights (drawn from --seed) of this configuration")
     gen.add_argument("--prompt-ids", action="append", help="comma-separated token ids; repeatable")
     gen.add_argument("--prompt-file", help="JSON file: a list of lists of token ids")
     gen.add_argument("--max-new-tokens", type=int, default=256)
@@ -113,11 +129,22 @@ def main(argv=None) -> None:
                          add_help=False)
     rep.add_argument("rest", nargs=argparse.REMAINDER)
 
+    ben = sub.add_parser("bench", help="decode and prefill throughput at the Qwen3-4B shape (bench.py)",
+                         add_help=False)
+    ben.add_argument("rest", nargs=argparse.REMAINDER)
+
     args = parser.parse_args(argv)
     if args.command == "generate":
         code = _generate(args)
     elif args.command == "random-model":
         code = _random_model(args)
+    elif args.command == "bench":
+        import runpy
+
+        script = Path(__file__).resolve().parent.parent / "bench.py"
+        sys.argv = [str(script), *args.rest]
+        runpy.run_path(str(script), run_name="__main__")
+        code = 0
     else:
         from .engine.replay import main as replay_main
 

@@ -176,3 +176,47 @@ def test_running_ahead_gives_the_tokens_of_the_tick_by_tick_engine(tmp, graphs):
         outputs.append([(r.output_ids, r.finish_reason) for r in greedy + cut + drawn])
         assert any(reason == "eos" for _, reason in outputs[-1])
     assert outputs[0] == outputs[1]
+
+
+def test_random_weights_straight_into_an_engine_and_the_command_line(tmp, tmp_path):
+    """Engine.from_random(config, seed) is the engine over the folder that the random-weights
+    mode writes from the same (config, seed); `main.py generate --random` prints its tokens."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    from pylon_amd.engine.engine import Engine
+    from pylon_amd.sampling import Sampling
+    from tests.helpers import CONFIGS, NORM_JITTER, SEEDS
+
+    folder = make_model_folder(tmp, "D", dtype="bfloat16")
+    prompt = random_tokens(CONFIGS["D"]["vocab_size"], 12, 3)
+    sampling = Sampling(max_new_tokens=10, temperature=0.0)
+    outputs = []
+    for make in (lambda: Engine.from_folder(folder, dtype="bfloat16", page_size=64, num_pages=4),
+                 lambda: Engine.from_random(CONFIGS["D"], SEEDS["D"], norm_jitter=NORM_JITTER["D"],
+                                            dtype="bfloat16", page_size=64, num_pages=4)):
+        engine = make()
+        try:
+            outputs.append(engine.generate([prompt], sampling)[0].output_ids)
+        finally:
+            engine.close()
+    assert outputs[0] == outputs[1] and len(outputs[0]) == 10
+    config_file = tmp_path / "config.json"
+    config_file.write_text(json.dumps(CONFIGS["D"]))
+    root = Path(__file__).resolve().parent.parent
+    done = subprocess.run(
+        [sys.executable, str(root / "main.py"), "generate", "--random", str(config_file), "--seed", str(SEEDS["D"]),
+         "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "10", "--temperature", "0",
+         "--page-size", "64", "--num-pages", "4"],
+        capture_output=True, text=True, timeout=120, cwd=str(tmp_path))
+    assert done.returncode == 0, done.stderr[-2000:]
+    line = json.loads(done.stdout.strip().splitlines()[-1])
+    # the command line draws unit norm weights (no jitter): the same as from_random without it
+    engine = Engine.from_random(CONFIGS["D"], SEEDS["D"], dtype="bfloat16", page_size=64, num_pages=4)
+    try:
+        want = engine.generate([prompt], sampling)[0].output_ids
+    finally:
+        engine.close()
+    assert line["output_ids"] == want and line["finish_reason"] == "length"
