@@ -8,7 +8,8 @@ the step function, then greedy sampling on the device and the copy of the chosen
 the host.  As in the engine's ticks, a step is queued before the host has read the ids of
 the step before it (they are fed back on the device), and every step's ids are read.  ``value`` is decoded tokens per second at the default batch of 8.  The same
 line carries the prefill of 2,048 tokens, the decode step's share of the HBM roofline,
-and decode rates at batch 1 and 64.
+decode rates at batch 1 and 64, and the batch-8 rate through the scheduler
+(``points.engine_b8``: queueing, admission and the prompts' prefill included).
 """
 from __future__ import annotations
 
@@ -152,6 +153,31 @@ def prefill_run(runner, cfg, repeats: int, seed: int):
     return times[len(times) // 2]
 
 
+def engine_run(runner, cfg, batch: int, seed: int) -> float:
+    """The same work through the scheduler: ``batch`` requests of PROMPT_LEN random ids and
+    NEW_TOKENS greedy tokens each, queued at once; generated tokens per second from the first
+    request's arrival to the last one's end (admission, the prompts' prefill, ticks, sampling
+    and the host's reading of every token included)."""
+    import numpy as np
+    import torch
+
+    from pylon_amd.config import PylonConfig
+    from pylon_amd.engine.engine import Engine
+    from pylon_amd.sampling import Sampling
+
+    rng = np.random.default_rng(seed)
+    prompts = [rng.integers(0, cfg.vocab_size, PROMPT_LEN).tolist() for _ in range(batch)]
+    engine = Engine(PylonConfig(max_batch_size=batch, max_queue_size=batch, page_size=PAGE_SIZE), runner=runner)
+    sampling = Sampling(max_new_tokens=NEW_TOKENS, temperature=0.0)
+    engine.generate(prompts[:1], Sampling(max_new_tokens=8, temperature=0.0))  # warm the batch-1 graph
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    results = engine.generate(prompts, sampling)
+    elapsed = time.perf_counter() - started
+    assert all(len(r.output_ids) == NEW_TOKENS for r in results)
+    return batch * NEW_TOKENS / elapsed
+
+
 def main() -> int:
     parser = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     parser.add_argument("--gpus", type=int, default=1)
@@ -225,6 +251,7 @@ def main() -> int:
             n = min(steps, 256)
             e, _ = decode_run(runner, cfg, batch, n, args.warmup, seed=3 + batch)
             points[f"decode_b{batch}"] = round(batch * n / e, 1)
+        points["engine_b8"] = round(engine_run(runner, cfg, batch=8, seed=9), 1)
         record["points"] = points
     print(json.dumps(record))
     return 0
