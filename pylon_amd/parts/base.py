@@ -13,7 +13,8 @@ norm          ``forward(x) -> y`` and ``add_forward(resid, delta, row_idx=None) 
               ``resid`` (unless ``row_idx`` picks rows), and its norm is returned in
               the activation dtype.
 position      ``rotary() -> (inv_freq, rotary_dim) | None`` for encodings applied by
-              rotating q and k, and ``check(max_position)``.
+              rotating q and k: float32 frequencies of the pairs ``(i, i + rotary_dim/2)``
+              of the first ``rotary_dim`` elements of a head; None encodes nothing.
 mixer         ``cache_requirement() -> KVRequirement | StateRequirement | None`` and
               ``forward(h, ctx, cache, stores) -> [tokens, hidden]`` (or partial sums
               ``[parts, tokens, hidden]`` in float32, see norm): ``cache`` is the

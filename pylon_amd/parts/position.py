@@ -30,13 +30,6 @@ class RotaryPosition(Part):
     def rotary(self) -> Optional[Tuple[torch.Tensor, int]]:
         return self.inv_freq, self.spec.rotary_dim
 
-    def check(self, max_position: int) -> None:
-        if self.spec.max_positions and max_position >= self.spec.max_positions:
-            raise ValueError(
-                f"position {max_position} is beyond the {self.spec.max_positions} positions "
-                "this model encodes"
-            )
-
 
 class NoPosition(Part):
     def __init__(self, spec: PositionSpec, *, dtype: torch.dtype, device) -> None:
@@ -44,9 +37,6 @@ class NoPosition(Part):
         self.spec = spec
 
     def rotary(self):
-        return None
-
-    def check(self, max_position: int) -> None:
         return None
 
 
