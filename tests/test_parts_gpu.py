@@ -68,9 +68,6 @@ def test_position_part_and_registry():
     inv, dim = rope.rotary()
     want = 1.0 / (np.float32(1e6) ** (np.arange(0, 32, 2, dtype=np.float32) / np.float32(32)))
     assert dim == 32 and np.allclose(inv.cpu().numpy(), want, rtol=1e-6)
-    rope.check(63)
-    with pytest.raises(ValueError, match="beyond"):
-        rope.check(64)
     assert build_part("position", PositionSpec("none"), dtype=torch.float32, device=DEV).rotary() is None
     with pytest.raises(ValueError, match="no position of kind 'alibi'"):
         build_part("position", PositionSpec("alibi"), dtype=torch.float32, device=DEV)
