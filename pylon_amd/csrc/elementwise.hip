@@ -93,24 +93,47 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, TX* x, const TD* __restrict
       wt[n] = (c < chunks) ? w4[c] : float4{0.f, 0.f, 0.f, 0.f};
     }
     if (dr) {
+      // Partial sums of the previous matrix product are added in a fixed order.  For the
+      // usual counts every load is issued before the first addition: a loop over a count
+      // only known at run time would wait for memory once per partial sum.
       const long long stride4 = delta_stride >> 2;
       float4 d[VEC];
+#define PYLON_SUM_PARTS(ND)                                                                   \
+  do {                                                                                        \
+    float4 e[ND][VEC];                                                                        \
+    _Pragma("unroll") for (int p = 0; p < ND; ++p) _Pragma("unroll") for (int n = 0; n < VEC; ++n) { \
+      const int c = threadIdx.x + n * blockDim.x;                                             \
+      e[p][n] = (c < chunks) ? load4(dr, c + p * stride4) : float4{0.f, 0.f, 0.f, 0.f};       \
+    }                                                                                         \
+    _Pragma("unroll") for (int n = 0; n < VEC; ++n) {                                         \
+      d[n] = e[0][n];                                                                         \
+      _Pragma("unroll") for (int p = 1; p < ND; ++p) {                                        \
+        d[n].x += e[p][n].x; d[n].y += e[p][n].y; d[n].z += e[p][n].z; d[n].w += e[p][n].w;   \
+      }                                                                                       \
+    }                                                                                         \
+  } while (0)
+      if (n_delta == 1) {
+        PYLON_SUM_PARTS(1);
+      } else if (n_delta == 2) {
+        PYLON_SUM_PARTS(2);
+      } else if (n_delta == 4) {
+        PYLON_SUM_PARTS(4);
+      } else if (n_delta == 8) {
+        PYLON_SUM_PARTS(8);
+      } else {
+        PYLON_SUM_PARTS(1);
+        for (int p = 1; p < n_delta; ++p) {
 #pragma unroll
-      for (int n = 0; n < VEC; ++n) {
-        const int c = threadIdx.x + n * blockDim.x;
-        d[n] = (c < chunks) ? load4(dr, c) : float4{0.f, 0.f, 0.f, 0.f};
-      }
-      // partial sums of the previous matrix product are added in a fixed order
-      for (int p = 1; p < n_delta; ++p) {
-#pragma unroll
-        for (int n = 0; n < VEC; ++n) {
-          const int c = threadIdx.x + n * blockDim.x;
-          if (c < chunks) {
-            const float4 e = load4(dr, c + p * stride4);
-            d[n].x += e.x; d[n].y += e.y; d[n].z += e.z; d[n].w += e.w;
+          for (int n = 0; n < VEC; ++n) {
+            const int c = threadIdx.x + n * blockDim.x;
+            if (c < chunks) {
+              const float4 e = load4(dr, c + p * stride4);
+              d[n].x += e.x; d[n].y += e.y; d[n].z += e.z; d[n].w += e.w;
+            }
           }
         }
       }
+#undef PYLON_SUM_PARTS
 #pragma unroll
       for (int n = 0; n < VEC; ++n) {
         held[n].x += d[n].x; held[n].y += d[n].y; held[n].z += d[n].z; held[n].w += d[n].w;
