@@ -22,9 +22,9 @@
 //
 // The kernel can also take over the step that precedes attention: given the raw q/k/v
 // projection instead of prepared queries, each workgroup first norms and rotates its
-// group's query heads (kept in LDS) and its key head, stores that key and its value head
-// at the token's cache slot, and only then reads the cache, the new key included.  One
-// launch and one pass over the projection less per layer.
+// group's query heads (kept in LDS) and its key head, and stores that key and its value
+// head at the token's cache slot.  The loads of older keys do not wait for that: the new
+// row is taken from LDS.  One launch and one pass over the projection less per layer.
 #include "common.h"
 #include "head_prepare.h"
 
@@ -33,7 +33,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 #define AD_MAX_GROUP 16
 #define AD_TILE 16   // keys per score tile
-#define AD_SUPER 64  // keys whose loads are in flight together (four score tiles)
+#define AD_SUPER 64  // most keys whose loads are in flight together (four score tiles)
 #define AD_MAX_WAVES 8
 
 // What the kernel needs to prepare q, k and v itself (PREP): the raw projection
@@ -73,7 +73,10 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
     const int* __restrict__ tok_row, const int* __restrict__ positions, int n_heads, int n_kv_heads,
     int page_size, int window, float scale, DecodePrep prep, float* __restrict__ partial) {
   constexpr int HD = EPL * 64;
-  constexpr int TILES = AD_SUPER / AD_TILE;
+  // keys whose loads are in flight together: 64 (four score tiles), or 32 where the
+  // fragments of 64 keys and the accumulators would not fit the registers
+  constexpr int SUPER = (EPL == 4 || GP >= 8) ? AD_SUPER / 2 : AD_SUPER;
+  constexpr int TILES = SUPER / AD_TILE;
   // per wave: probabilities of the keys in flight; then the waves' partial results
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int n_waves = blockDim.x / PYLON_WAVE;
@@ -108,6 +111,10 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
   int k_end = k_begin + per_wave;
   if (k_end > c_end) k_end = c_end;
 
+  // PREP: the token's own key and value, as they go into the cache, also stay in LDS: the
+  // loads of old keys need not wait for those stores, and the new row is taken from here.
+  uint16_t* kv_new = reinterpret_cast<uint16_t*>(reinterpret_cast<float*>(q_lds + GP * HD) + n_waves * HD);
+  bool stored_new = false;
   if constexpr (PREP) {
     // 512/head_dim heads per wave at a time: the group's query heads into LDS, then this
     // key head and this value head into the token's cache slot.
@@ -118,6 +125,7 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
     // the new key and value are stored by the one workgroup whose keys include them
     const int slot = (prep.slot_map != nullptr && holds_last) ? prep.slot_map[t] : -1;
     const int jobs = group + (slot >= 0 ? 2 : 0);
+    stored_new = slot >= 0;
     const int j = lane % LPH;
     // job -> where its head lies in the projection's row
     auto source = [&](int job) {
@@ -150,11 +158,47 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
       } else if (valid) {
         uint16_t* dst = (is_key ? k_cache : v_cache) + (static_cast<size_t>(slot) * n_kv_heads + kvh) * HD + 8 * j;
         store8_bf16(dst, v);
+        store8_bf16(kv_new + (is_key ? 0 : HD) + 8 * j, v);
       }
     }
-    // The barrier orders the workgroup's stores before its loads: every wave sees the new
-    // key and value in the cache and the queries in LDS.
-    __syncthreads();
+  }
+
+  // Every load of 64 keys and values is issued before the first is used.  Lane `lane`
+  // owns key BASE + lane for the value rows; for the score tiles, row `col` of tile `kt`
+  // is key BASE + 16*kt + col.  Keys past the end repeat the last key.  Values: LPK lanes
+  // read one key's row, 8 elements each; KPI keys per load instruction.
+  constexpr int LPK = HD / 8;             // lanes that share one key's value row
+  constexpr int KPI = PYLON_WAVE / LPK;   // keys per value load instruction
+  const int vkey = lane / LPK, vchunk = lane % LPK;
+  bf16x8 kf[TILES][KSTEPS];
+  uint4 vv[SUPER / KPI];
+#define AD_LOAD(BASE)                                                                                  \
+  do {                                                                                                 \
+    const int my_key = ((BASE) + lane < k_end) ? (BASE) + lane : k_end - 1;                            \
+    const int my_page = my_key / page_size;                                                            \
+    int page_id = __shfl(table_entry, my_page & (PYLON_WAVE - 1), PYLON_WAVE);                         \
+    if (my_page >= PYLON_WAVE) page_id = table[my_page];                                               \
+    const int my_phys = page_id * page_size + my_key % page_size;                                      \
+    _Pragma("unroll") for (int kt = 0; kt < TILES; ++kt) {                                             \
+      const int phys = __shfl(my_phys, kt * 16 + col, PYLON_WAVE);                                     \
+      const uint16_t* krow = k_cache + (static_cast<size_t>(phys) * n_kv_heads + kvh) * HD;            \
+      _Pragma("unroll") for (int ks = 0; ks < KSTEPS; ++ks)                                            \
+          kf[kt][ks] = *reinterpret_cast<const bf16x8*>(krow + ks * 32 + grp * 8);                     \
+    }                                                                                                  \
+    _Pragma("unroll") for (int i = 0; i < SUPER / KPI; ++i) {                                       \
+      const int pk = __shfl(my_phys, i * KPI + vkey, PYLON_WAVE);                                      \
+      const uint16_t* vrow = v_cache + (static_cast<size_t>(pk) * n_kv_heads + kvh) * HD;              \
+      vv[i] = *reinterpret_cast<const uint4*>(vrow + vchunk * 8);                                      \
+    }                                                                                                  \
+  } while (0)
+
+  if (k_begin < k_end) AD_LOAD(k_begin);  // on their way while the queries settle in LDS
+  if constexpr (PREP) {
+    // Only LDS has to be in order across this barrier (the queries, the new key and value):
+    // the loads above and the stores into the cache stay in flight.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
   }
   // query fragments: column `col` is head kvh*group + col of the token
   bf16x8 qf[KSTEPS];
@@ -174,39 +218,30 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
   }
 
   float m_run = -INFINITY, l_run = 0.f;  // for head `col` (same in the 4 lanes that share it)
-  constexpr int LPK = HD / 8;             // lanes that share one key's value row
-  constexpr int KPI = PYLON_WAVE / LPK;   // keys per value load instruction
-  const int vkey = lane / LPK, vchunk = lane % LPK;
   float acc[GP][8];  // elements vchunk*8 .. +7 over this lane's keys; rows past `group` unused
 #pragma unroll
   for (int h = 0; h < GP; ++h)
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
 
-  for (int base = k_begin; base < k_end; base += AD_SUPER) {
-    // Every load of these 64 keys and values is issued before the first is used.
-    // Lane `lane` owns key base + lane for the value rows; for the score tiles, row `col`
-    // of tile `kt` is key base + 16*kt + col.  Keys past the end repeat the last key.
-    const int my_key = (base + lane < k_end) ? base + lane : k_end - 1;
-    const int my_page = my_key / page_size;
-    int page_id = __shfl(table_entry, my_page & (PYLON_WAVE - 1), PYLON_WAVE);
-    if (my_page >= PYLON_WAVE) page_id = table[my_page];
-    const int my_phys = page_id * page_size + my_key % page_size;
-    bf16x8 kf[TILES][KSTEPS];
+  // this wave's keys end with the token's own, which the cache may not hold yet
+  const bool patch = PREP && stored_new && k_end == pos + 1;
+  for (int base = k_begin; base < k_end; base += SUPER) {
+    if (base != k_begin) AD_LOAD(base);
+    if (patch && base + SUPER >= k_end) {
+      // rows of the new key (and of the lanes past the end, which repeat it) come from LDS
 #pragma unroll
-    for (int kt = 0; kt < TILES; ++kt) {
-      const int phys = __shfl(my_phys, kt * 16 + col, PYLON_WAVE);
-      const uint16_t* krow = k_cache + (static_cast<size_t>(phys) * n_kv_heads + kvh) * HD;
+      for (int kt = 0; kt < TILES; ++kt) {
+        if (base + kt * 16 + col >= pos) {
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) kf[kt][ks] = *reinterpret_cast<const bf16x8*>(krow + ks * 32 + grp * 8);
-    }
-    // values: LPK lanes read one key's row, 8 elements each; KPI keys per load instruction
-    uint4 vv[AD_SUPER / KPI];
+          for (int ks = 0; ks < KSTEPS; ++ks)
+            kf[kt][ks] = *reinterpret_cast<const bf16x8*>(kv_new + ks * 32 + grp * 8);
+        }
+      }
 #pragma unroll
-    for (int i = 0; i < AD_SUPER / KPI; ++i) {
-      const int pk = __shfl(my_phys, i * KPI + vkey, PYLON_WAVE);
-      const uint16_t* vrow = v_cache + (static_cast<size_t>(pk) * n_kv_heads + kvh) * HD;
-      vv[i] = *reinterpret_cast<const uint4*>(vrow + vchunk * 8);
+      for (int i = 0; i < SUPER / KPI; ++i) {
+        if (base + i * KPI + vkey >= pos) vv[i] = *reinterpret_cast<const uint4*>(kv_new + HD + vchunk * 8);
+      }
     }
 
     floatx4 s[TILES];
@@ -255,7 +290,7 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
     }
     // keys past the end weigh 0 and their value row is the (finite) last key's
 #pragma unroll
-    for (int i = 0; i < AD_SUPER / KPI; ++i) {
+    for (int i = 0; i < SUPER / KPI; ++i) {
       const uint32_t w[4] = {vv[i].x, vv[i].y, vv[i].z, vv[i].w};
       float v[8];
 #pragma unroll
@@ -328,6 +363,8 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
   }
 }
 
+#undef AD_LOAD
+
 // One wave per (token, query head) merges the partial results of the cuts, in their order.
 template <int EPL>
 __global__ __launch_bounds__(PYLON_WAVE) void attention_decode_merge_kernel(
@@ -357,7 +394,9 @@ __global__ __launch_bounds__(PYLON_WAVE) void attention_decode_merge_kernel(
 
 static size_t decode_lds_bytes(int n_waves, int gp, int head_dim, bool prep) {
   return sizeof(float) * decode_lds_floats(n_waves, gp, head_dim) +
-         (prep ? sizeof(uint16_t) * static_cast<size_t>(gp) * head_dim + sizeof(float) * n_waves * head_dim : 0);
+         (prep ? sizeof(uint16_t) * static_cast<size_t>(gp) * head_dim + sizeof(float) * n_waves * head_dim +
+                     sizeof(uint16_t) * 2 * head_dim
+               : 0);
 }
 
 template <int EPL, bool PREP>
