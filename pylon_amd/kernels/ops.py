@@ -207,7 +207,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
 
 DECODE_HEAD_DIMS = (64, 128, 256)
-DECODE_MAX_TOKENS = 64
+DECODE_MAX_TOKENS = 1024  # beyond this many single-token rows the prefill kernel's tiling takes over
 
 
 def decode_attention_ok(q: torch.Tensor, k_cache: torch.Tensor) -> bool:
@@ -221,8 +221,8 @@ def decode_attention_ok(q: torch.Tensor, k_cache: torch.Tensor) -> bool:
 def decode_splits(tokens: int, n_kv_heads: int, max_len: Optional[int]) -> int:
     """Wavefronts (1, 2, 4 or 8) that share the keys of one (token, key/value head):
     ranges of about 64 keys (one batch of loads per wave) while the launch stays within a
-    few thousand waves.  Without a known length (graph capture) the count depends on the
-    batch size only."""
+    few thousand waves.  ``max_len`` is the most keys a workgroup gets (an upper bound
+    under graph capture)."""
     waves = 8
     while waves > 1 and tokens * n_kv_heads * waves > 4096:
         waves //= 2

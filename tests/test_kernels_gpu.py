@@ -356,6 +356,25 @@ def test_attention_decode(ops, geom, n_splits, n_cuts):
     assert torch.equal(same, got)
 
 
+def test_attention_decode_for_a_large_batch(ops):
+    """Three hundred single-token rows in one launch agree with the general kernel."""
+    nh, nkv, hd, page, tokens = 8, 2, 64, 16, 300
+    gen = torch.Generator().manual_seed(77)
+    lengths = torch.randint(1, 200, (tokens,), generator=gen)
+    width = int(-(-lengths.max() // page))
+    table = torch.randperm(tokens * width, generator=gen).to(torch.int32).reshape(tokens, width)
+    kc = rnd((tokens * width, page, nkv, hd), 78, torch.bfloat16).to(DEV)
+    vc = rnd((tokens * width, page, nkv, hd), 79, torch.bfloat16).to(DEV)
+    q = rnd((tokens, nh, hd), 80, torch.bfloat16).to(DEV)
+    pos = (lengths - 1).to(torch.int32).to(DEV)
+    rows = torch.arange(tokens, dtype=torch.int32, device=DEV)
+    want = ops.paged_attention(q, kc, vc, table.to(DEV), rows, pos, page_size=page, window=None, scale=0.125)
+    splits = ops.decode_splits(tokens, nkv, int(lengths.max()))
+    got = ops.attention_decode(q, kc, vc, table.to(DEV), None, pos, page_size=page, window=None, scale=0.125,
+                               n_splits=splits)
+    assert np.abs(f64(got) - f64(want)).max() <= tol(torch.bfloat16, 1.0)
+
+
 @pytest.mark.parametrize("geom", [(8, 2, 128, 64, None), (4, 4, 64, 16, None), (12, 2, 128, 32, 100),
                                   (5, 1, 256, 16, None), (3, 3, 64, 256, 37), (16, 1, 128, 64, None),
                                   (8, 4, 128, 48, None), (6, 2, 64, 80, 90)])
