@@ -220,3 +220,42 @@ def test_random_weights_straight_into_an_engine_and_the_command_line(tmp, tmp_pa
     finally:
         engine.close()
     assert line["output_ids"] == want and line["finish_reason"] == "length"
+
+
+def test_a_random_workload_gives_the_same_tokens_in_every_mode_of_the_engine(tmp):
+    """Fifty requests of random lengths, greedy and seeded sampling, half of them with a stop
+    token that they really meet, through the scheduler with few pages and slots: tick by
+    tick or running ahead, kernel by kernel or from graphs, every request's tokens are the
+    same (float32 kernels do not depend on what shares a batch)."""
+    from pylon_amd.engine.engine import Engine
+    from pylon_amd.sampling import Sampling
+
+    folder = make_model_folder(tmp, "D", dtype="float32", std=0.08)
+    cfg, _ = read_folder(folder)
+    rng = np.random.default_rng(5)
+    requests = []
+    for i in range(50):
+        prompt = rng.integers(0, cfg["vocab_size"], int(rng.integers(1, 260))).tolist()
+        sampling = Sampling(max_new_tokens=int(rng.integers(1, 40)), temperature=float(rng.choice([0.0, 0.8])),
+                            top_p=0.9, seed=i)
+        requests.append((prompt, sampling))
+
+    def run(stops, **options):
+        engine = Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=60, max_batch_size=6,
+                                    prefill_chunk_size=64, max_queue_size=64, **options)
+        try:
+            futures = [engine.enqueue(p, stop, s, f"r{i}") for i, ((p, s), stop) in enumerate(zip(requests, stops))]
+            engine.run_until_idle()
+            results = [f.result(timeout=0) for f in futures]
+        finally:
+            engine.close()
+        assert engine.runner.manager.free_pages == 60
+        engine.runner.manager.check()
+        return [(r.output_ids, r.finish_reason) for r in results]
+
+    free = run([None] * len(requests))
+    stops = [out[4] if i % 2 == 0 and len(out) > 4 else None for i, (out, _) in enumerate(free)]
+    base = run(stops, run_ahead=False)
+    assert sum(reason == "eos" for _, reason in base) >= 10
+    for options in (dict(run_ahead=True), dict(run_ahead=False, cuda_graphs=True), dict(run_ahead=True, cuda_graphs=True)):
+        assert run(stops, **options) == base, options
