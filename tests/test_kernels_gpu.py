@@ -306,7 +306,7 @@ def test_attention_decode(ops, geom, n_splits, n_cuts):
     workgroups (n_cuts): also with more shares than a short request has keys."""
     nh, nkv, hd, page, window = geom
     dtype = torch.bfloat16
-    lengths = [1, 15, 16, 17, 65, 300, 2 * page + 1, 700]
+    lengths = [1, 15, 16, 17, 65, 300, 2 * page + 1, 700, 70 * page + 3]  # the last: a table of over 64 pages
     n_pages = sum(-(-n // page) for n in lengths) + 2
     perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(40)).tolist()
     width = max(-(-n // page) for n in lengths)
