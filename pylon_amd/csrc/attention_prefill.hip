@@ -37,11 +37,11 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 // is a power of two, so a key's page and offset are a shift and a mask (a division by a
 // run-time number costs some twenty instructions, eight times per thread and block).
 template <int HD, int QT, bool POW2>
-__global__ __launch_bounds__(256) void attention_prefill_kernel(
+__global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
-    const int* __restrict__ tiles, int n_heads, int n_kv_heads, int group, int page_size, int window,
-    float scale) {
+    const int* __restrict__ tiles, int n_tiles, int per_wg, int n_heads, int n_kv_heads, int group,
+    int page_size, int window, float scale) {
   constexpr int KS = HD / 32;        // 32-wide steps along the head for a score tile
   constexpr int DT = HD / 16;        // 16-wide output tiles along the head
   constexpr int KSTR = HD + 8;       // row stride of the key tile (elements)
@@ -56,7 +56,12 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   const int lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, grp = lane >> 4;
   const int kvh = blockIdx.y;
-  const int* td = tiles + blockIdx.x * 4;
+  // A workgroup takes per_wg tiles one after the other (the host pairs a long one with a
+  // short one, so that every workgroup has about the same number of key blocks to walk).
+  for (int part = 0; part < per_wg; ++part) {
+  const int tile = blockIdx.x * per_wg + part;
+  if (tile >= n_tiles) break;
+  const int* td = tiles + tile * 4;
   const int tok0 = td[0], ntok = td[1], trow = td[2], pos0 = td[3];
   const int* table = block_table + static_cast<size_t>(trow) * table_width;
   const int kv_last = pos0 + ntok - 1;
@@ -286,6 +291,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
       }
     }
   }
+  __syncthreads();  // LDS (the page table, the last block) is free for the next tile
+  }
 }
 
 // tiles: [n_tiles, 4] = (index of the tile's first token in q/out, its token count, its row of
@@ -295,7 +302,9 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 extern "C" int pylon_attention_prefill(void* out, const void* q, const void* k_cache, const void* v_cache,
                                        const int* block_table, int table_width, const int* tiles,
                                        int n_tiles, int n_heads, int n_kv_heads, int head_dim,
-                                       int page_size, int window, float scale, int rows, hipStream_t stream) {
+                                       int page_size, int window, float scale, int rows, int per_wg,
+                                       hipStream_t stream) {
+  PYLON_REQUIRE(per_wg >= 1 && per_wg <= 8, "attention_prefill: 1..8 tiles per workgroup, got %d", per_wg);
   PYLON_REQUIRE(rows == 64 || rows == 128, "attention_prefill: 64 or 128 query rows per workgroup, got %d", rows);
   PYLON_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "attention_prefill: %d query heads cannot be grouped over %d key/value heads", n_heads,
@@ -310,18 +319,18 @@ extern "C" int pylon_attention_prefill(void* out, const void* q, const void* k_c
   PYLON_REQUIRE(n_kv_heads <= 65535, "attention_prefill: too many key/value heads for one launch");
   if (n_tiles == 0) return 0;
   const int group = n_heads / n_kv_heads;
-  dim3 grid(n_tiles, n_kv_heads), block(256);
+  dim3 grid((n_tiles + per_wg - 1) / per_wg, n_kv_heads), block(256);
   const bool pow2 = (page_size & (page_size - 1)) == 0;
 #define GO(HD, QT)                                                                                       \
   do {                                                                                                   \
     if (pow2)                                                                                            \
       hipLaunchKernelGGL((attention_prefill_kernel<HD, QT, true>), grid, block, 0, stream, (uint16_t*)out, \
                          (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache,         \
-                         block_table, table_width, tiles, n_heads, n_kv_heads, group, page_size, window, scale); \
+                         block_table, table_width, tiles, n_tiles, per_wg, n_heads, n_kv_heads, group, page_size, window, scale); \
     else                                                                                                 \
       hipLaunchKernelGGL((attention_prefill_kernel<HD, QT, false>), grid, block, 0, stream, (uint16_t*)out, \
                          (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache,         \
-                         block_table, table_width, tiles, n_heads, n_kv_heads, group, page_size, window, scale); \
+                         block_table, table_width, tiles, n_tiles, per_wg, n_heads, n_kv_heads, group, page_size, window, scale); \
   } while (0)
   if (rows == 64) {
     if (head_dim == 64) GO(64, 1);
