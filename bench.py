@@ -2,6 +2,7 @@
 and uniform-random token ids, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+                    [--shape 4b|8b|32b] [--prompt-len N]
 
 A "step" is one decode step: one token for each of ``batch`` running requests through
 the step function, then greedy sampling on the device and the copy of the chosen ids to
@@ -10,6 +11,8 @@ the step before it (they are fed back on the device), and every step's ids are r
 line carries the prefill of 2,048 tokens, the decode step's share of the HBM roofline,
 decode rates at batch 1 and 64, and the batch-8 rate through the scheduler
 (``points.engine_b8``: queueing, admission and the prompts' prefill included).
+``--shape`` and ``--prompt-len`` measure the same at the Qwen3-8B and 32B layer sizes and
+at longer contexts; the default run is the 4B shape with 128-token prompts.
 """
 from __future__ import annotations
 
@@ -33,33 +36,43 @@ SHAPE_4B = dict(
     head_dim=128, intermediate_size=9728, vocab_size=151936, rope_theta=5000000.0,
     rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=8192,
 )
-CONTEXT_LENGTH = 8192
+SHAPE_8B = dict(
+    num_hidden_layers=36, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+    head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1000000.0,
+    rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768,
+)
+SHAPE_32B = dict(
+    num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8,
+    head_dim=128, intermediate_size=25600, vocab_size=151936, rope_theta=1000000.0,
+    rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=32768,
+)
+SHAPES = {"4b": SHAPE_4B, "8b": SHAPE_8B, "32b": SHAPE_32B}
 PAGE_SIZE = 256
 PROMPT_LEN = 128
 NEW_TOKENS = 512
 PREFILL_TOKENS = 2048
 
 
-def config_json(layers: int) -> dict:
-    cfg = dict(SHAPE_4B, num_hidden_layers=layers)
+def config_json(shape: dict, layers: int) -> dict:
+    cfg = dict(shape, num_hidden_layers=layers)
     cfg.update(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_act="silu")
     return cfg
 
 
-def build_runner(layers: int, dtype: str, max_requests: int, num_pages: int, graphs: bool):
+def build_runner(shape: dict, layers: int, dtype: str, max_requests: int, num_pages: int, graphs: bool):
     import torch
 
     from pylon_amd.config import resolve
     from pylon_amd.engine import Model, Runner, resolve_dtype
 
-    raw = config_json(layers)
+    raw = config_json(shape, layers)
     arch = resolve(raw)
     cfg = arch.parse_config(raw)
     model = Model(arch.model_spec(cfg), dtype=resolve_dtype(dtype), device="cuda:0")
     model.init_random(seed=0)
     runner = Runner(model, page_size=PAGE_SIZE, num_pages=num_pages, max_requests=max_requests)
     if graphs:
-        runner.enable_graphs(max_requests, max_tokens_per_request=CONTEXT_LENGTH)
+        runner.enable_graphs(max_requests, max_tokens_per_request=shape["max_position_embeddings"])
     torch.cuda.synchronize()
     return runner, cfg
 
@@ -83,8 +96,35 @@ def linear_flops_per_token(cfg) -> float:
     return 2.0 * cfg.num_hidden_layers * per_layer
 
 
-def decode_run(runner, cfg, batch: int, steps: int, warmup: int, seed: int):
-    """Prefill ``batch`` prompts of PROMPT_LEN random ids, then time ``steps`` decode steps."""
+def feed_prompts(runner, sampler, seqs, prompts) -> None:
+    """The prompts through the step function in steps of at most PREFILL_TOKENS tokens, cut as
+    the scheduler cuts them (short prompts side by side, a long one in portions); the first
+    new token of each request is chosen on the device."""
+    from pylon_amd.engine import StepEntry
+    from pylon_amd.sampling import Sampling
+
+    fed = [0] * len(seqs)
+    at = 0
+    while at < len(seqs):
+        entries, budget = [], PREFILL_TOKENS
+        while at < len(seqs) and budget > 0:
+            take = min(budget, len(prompts[at]) - fed[at])
+            last = fed[at] + take == len(prompts[at])
+            entries.append(StepEntry(seqs[at], prompts[at][fed[at]: fed[at] + take], [take - 1] if last else []))
+            fed[at] += take
+            budget -= take
+            if not last:
+                break
+            at += 1
+        out = runner.step(entries)
+        wanted = sum(len(e.want) for e in entries)
+        if wanted:
+            greedy = [(Sampling(temperature=0.0), 0)] * wanted
+            sampler.launch(out, greedy, chosen=runner.chosen, place=runner.logit_slots).result()
+
+
+def decode_run(runner, cfg, batch: int, steps: int, warmup: int, seed: int, prompt_len: int = PROMPT_LEN):
+    """Prefill ``batch`` prompts of ``prompt_len`` random ids, then time ``steps`` decode steps."""
     import numpy as np
     import torch
 
@@ -95,13 +135,8 @@ def decode_run(runner, cfg, batch: int, steps: int, warmup: int, seed: int):
     greedy = [(Sampling(temperature=0.0), 0)] * batch
     rng = np.random.default_rng(seed)
     seqs = [runner.open(f"b{batch}-{i}") for i in range(batch)]
-    prompts = [rng.integers(0, cfg.vocab_size, PROMPT_LEN).tolist() for _ in range(batch)]
-    # prompts in portions of up to 2048 tokens, as the scheduler would cut them
-    per_step = max(1, PREFILL_TOKENS // PROMPT_LEN)
-    for lo in range(0, batch, per_step):
-        part = list(range(lo, min(batch, lo + per_step)))
-        out = runner.step([StepEntry(seqs[i], prompts[i], [PROMPT_LEN - 1]) for i in part])
-        sampler.launch(out, greedy[: len(part)], chosen=runner.chosen, place=runner.logit_slots).result()
+    prompts = [rng.integers(0, cfg.vocab_size, prompt_len).tolist() for _ in range(batch)]
+    feed_prompts(runner, sampler, seqs, prompts)
 
     entries = [StepEntry(seqs[i], [PENDING], [0]) for i in range(batch)]
     produced = []
@@ -153,8 +188,8 @@ def prefill_run(runner, cfg, repeats: int, seed: int):
     return times[len(times) // 2]
 
 
-def engine_run(runner, cfg, batch: int, seed: int) -> float:
-    """The same work through the scheduler: ``batch`` requests of PROMPT_LEN random ids and
+def engine_run(runner, cfg, batch: int, seed: int, prompt_len: int = PROMPT_LEN) -> float:
+    """The same work through the scheduler: ``batch`` requests of ``prompt_len`` random ids and
     NEW_TOKENS greedy tokens each, queued at once; generated tokens per second from the first
     request's arrival to the last one's end (admission, the prompts' prefill, ticks, sampling
     and the host's reading of every token included)."""
@@ -166,7 +201,7 @@ def engine_run(runner, cfg, batch: int, seed: int) -> float:
     from pylon_amd.sampling import Sampling
 
     rng = np.random.default_rng(seed)
-    prompts = [rng.integers(0, cfg.vocab_size, PROMPT_LEN).tolist() for _ in range(batch)]
+    prompts = [rng.integers(0, cfg.vocab_size, prompt_len).tolist() for _ in range(batch)]
     engine = Engine(PylonConfig(max_batch_size=batch, max_queue_size=batch, page_size=PAGE_SIZE), runner=runner)
     sampling = Sampling(max_new_tokens=NEW_TOKENS, temperature=0.0)
     engine.generate(prompts[:1], Sampling(max_new_tokens=8, temperature=0.0))  # warm the batch-1 graph
@@ -184,7 +219,9 @@ def main() -> int:
     parser.add_argument("--steps", type=int, default=NEW_TOKENS)
     parser.add_argument("--warmup", type=int, default=16)
     parser.add_argument("--batch", type=int, default=8)
-    parser.add_argument("--layers", type=int, default=SHAPE_4B["num_hidden_layers"])
+    parser.add_argument("--shape", choices=sorted(SHAPES), default="4b", help="layer sizes (default: Qwen3-4B)")
+    parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has")
+    parser.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens cached before decoding starts")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
@@ -201,19 +238,30 @@ def main() -> int:
         print("bench.py: A GPU is required.", file=sys.stderr)
         return 1
 
-    max_batch = max(64, args.batch)
-    pages_per_request = CONTEXT_LENGTH // PAGE_SIZE
-    runner, cfg = build_runner(args.layers, args.dtype, max_requests=max_batch,
+    shape = SHAPES[args.shape]
+    layers = args.layers or shape["num_hidden_layers"]
+    context_length = shape["max_position_embeddings"]
+    prompt_len = args.prompt_len
+    steps = min(args.steps, context_length - prompt_len - args.warmup)
+    max_batch = args.batch if args.no_points else max(64, args.batch)
+    # The pool holds a whole context for every request where that stays under a third of the
+    # card's memory, else what the longest run here needs.
+    element = 2 if args.dtype == "bfloat16" else 4
+    page_bytes = 2 * layers * PAGE_SIZE * shape["num_key_value_heads"] * shape["head_dim"] * element
+    pages_per_request = context_length // PAGE_SIZE
+    if max_batch * pages_per_request * page_bytes > 100e9:
+        longest = max(prompt_len + steps + args.warmup + 1, PREFILL_TOKENS)
+        pages_per_request = -(-longest // PAGE_SIZE) + 1
+    runner, cfg = build_runner(shape, layers, args.dtype, max_requests=max_batch,
                                num_pages=max_batch * pages_per_request, graphs=not args.no_graphs)
     dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
-    steps = min(args.steps, CONTEXT_LENGTH - PROMPT_LEN - args.warmup)
     if args.prefill_only:
         seconds = prefill_run(runner, cfg, repeats=5, seed=2)
         print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
                                       "ms": round(1e3 * seconds, 3)}}))
         return 0
 
-    elapsed, mean_context = decode_run(runner, cfg, args.batch, steps, args.warmup, seed=1)
+    elapsed, mean_context = decode_run(runner, cfg, args.batch, steps, args.warmup, seed=1, prompt_len=prompt_len)
     ms_per_step = 1e3 * elapsed / steps
     value = args.batch * steps / elapsed
     per_token = runner.manager.bytes_per_token
@@ -221,17 +269,17 @@ def main() -> int:
     achieved = step_bytes / (elapsed / steps)
 
     record = {
-        "metric": "decode tokens/s, Qwen3-4B shape, batch 8, 128-token prompts",
+        "metric": f"decode tokens/s, Qwen3-{args.shape.upper()} shape, batch {args.batch}, {prompt_len}-token prompts",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dtype_key, "data": "synthetic",
         "config": {
-            "model": "qwen3-4b-shape-random", "layers": args.layers,
-            "layers_full": SHAPE_4B["num_hidden_layers"], "hidden": cfg.hidden_size,
+            "model": f"qwen3-{args.shape}-shape-random", "layers": layers,
+            "layers_full": shape["num_hidden_layers"], "hidden": cfg.hidden_size,
             "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
-            "global_batch": args.batch, "seq_len": PROMPT_LEN, "new_tokens": steps,
-            "context_length": CONTEXT_LENGTH, "page_size": PAGE_SIZE, "prefill_tokens": PREFILL_TOKENS,
+            "global_batch": args.batch, "seq_len": prompt_len, "new_tokens": steps,
+            "context_length": context_length, "page_size": PAGE_SIZE, "prefill_tokens": PREFILL_TOKENS,
             "hip_graphs": runner.graphs is not None, "parallelism": "single-gpu",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_BYTES_PER_S / 1e9,
@@ -249,9 +297,9 @@ def main() -> int:
         points = {}
         for batch in (1, 64):
             n = min(steps, 256)
-            e, _ = decode_run(runner, cfg, batch, n, args.warmup, seed=3 + batch)
+            e, _ = decode_run(runner, cfg, batch, n, args.warmup, seed=3 + batch, prompt_len=prompt_len)
             points[f"decode_b{batch}"] = round(batch * n / e, 1)
-        points["engine_b8"] = round(engine_run(runner, cfg, batch=8, seed=9), 1)
+        points["engine_b8"] = round(engine_run(runner, cfg, batch=8, seed=9, prompt_len=prompt_len), 1)
         record["points"] = points
     print(json.dumps(record))
     return 0
