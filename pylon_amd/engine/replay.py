@@ -66,6 +66,8 @@ def main(argv=None) -> int:
         entries = []
         for item in record.get("entries", []):
             rid = item["id"]
+            if not item["tokens"]:
+                continue  # nothing to run for this request in this step
             seq = live.get(rid)
             if seq is None:
                 seq = live[rid] = runner.open(rid)
