@@ -33,10 +33,12 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{lo, hi}, bf16x2));
 }
 
-// QT: 16-row query tiles per wave (1: 64 rows per workgroup, 2: 128).  POW2: the page size
-// is a power of two, so a key's page and offset are a shift and a mask (a division by a
-// run-time number costs some twenty instructions, eight times per thread and block).
-template <int HD, int QT, bool POW2>
+// QT: 16-row query tiles per wave (1: 64 rows per workgroup, 2: 128).  PAGING says how a
+// key's place in the cache is found: 0 by a division by the page size (some twenty
+// instructions, eight times per thread and block), 1 by a shift and a mask (the page size is
+// a power of two), 2 once per block of 64 keys, which then lies inside one page (a power of
+// two of at least 64).
+template <int HD, int QT, int PAGING>
 __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
@@ -79,33 +81,57 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   u32x4 kreg[KP], vreg[VC][4];
   const int page_shift = __ffs(page_size) - 1, page_mask = page_size - 1;
   const size_t row_elems = static_cast<size_t>(n_kv_heads) * HD;
+  const unsigned row_elems32 = n_kv_heads * HD;  // a block of 64 rows spans far less than 4 GiB
   const uint16_t* k_head = k_cache + static_cast<size_t>(kvh) * HD;
   const uint16_t* v_head = v_cache + static_cast<size_t>(kvh) * HD;
 #define AP_SLOT(J, PHYS)                                                                               \
   do {                                                                                                 \
-    const int pg = POW2 ? (J) >> page_shift : (J) / page_size;                                         \
-    const int off = POW2 ? (J) & page_mask : (J) - pg * page_size;                                     \
+    const int pg = PAGING ? (J) >> page_shift : (J) / page_size;                                       \
+    const int off = PAGING ? (J) & page_mask : (J) - pg * page_size;                                   \
     PHYS = table_lds[pg] * page_size + off;                                                            \
   } while (0)
 #define AP_FETCH(KB)                                                                                   \
   do {                                                                                                 \
-    _Pragma("unroll") for (int i = 0; i < KP; ++i) {                                                   \
-      const int idx = i * 256 + tid;                                                                   \
-      const int key = idx / CHUNKS, chunk = idx - key * CHUNKS;                                        \
-      const int j = ((KB) + key < kv_last) ? (KB) + key : kv_last;                                     \
-      int phys;                                                                                        \
-      AP_SLOT(j, phys);                                                                                \
-      kreg[i] = *reinterpret_cast<const u32x4*>(k_head + static_cast<size_t>(phys) * row_elems + chunk * 8); \
-    }                                                                                                  \
-    _Pragma("unroll") for (int i = 0; i < VC; ++i) {                                                   \
-      const int idx = i * 256 + tid;                                                                   \
-      const int chunk = idx >> 4, quad = idx & 15;                                                     \
-      if (chunk < CHUNKS) {                                                                            \
-        _Pragma("unroll") for (int p = 0; p < 4; ++p) {                                                \
-          const int j = ((KB) + 4 * quad + p < kv_last) ? (KB) + 4 * quad + p : kv_last;               \
-          int phys;                                                                                    \
-          AP_SLOT(j, phys);                                                                            \
-          vreg[i][p] = *reinterpret_cast<const u32x4*>(v_head + static_cast<size_t>(phys) * row_elems + chunk * 8); \
+    if constexpr (PAGING == 2) {                                                                       \
+      const int page_row = table_lds[(KB) >> page_shift] * page_size + ((KB) & page_mask);             \
+      const uint16_t* k_block = k_head + static_cast<size_t>(page_row) * row_elems;                    \
+      const uint16_t* v_block = v_head + static_cast<size_t>(page_row) * row_elems;                    \
+      const unsigned last = kv_last - (KB);                                                            \
+      _Pragma("unroll") for (int i = 0; i < KP; ++i) {                                                 \
+        const unsigned idx = i * 256 + tid;                                                            \
+        const unsigned key = idx / CHUNKS, chunk = idx - key * CHUNKS;                                 \
+        const unsigned j = key < last ? key : last;                                                    \
+        kreg[i] = *reinterpret_cast<const u32x4*>(k_block + (j * row_elems32 + chunk * 8));            \
+      }                                                                                                \
+      _Pragma("unroll") for (int i = 0; i < VC; ++i) {                                                 \
+        const unsigned idx = i * 256 + tid;                                                            \
+        const unsigned chunk = idx >> 4, quad = idx & 15;                                              \
+        if (chunk < CHUNKS) {                                                                          \
+          _Pragma("unroll") for (int p = 0; p < 4; ++p) {                                              \
+            const unsigned j = 4 * quad + p < last ? 4 * quad + p : last;                              \
+            vreg[i][p] = *reinterpret_cast<const u32x4*>(v_block + (j * row_elems32 + chunk * 8));     \
+          }                                                                                            \
+        }                                                                                              \
+      }                                                                                                \
+    } else {                                                                                           \
+      _Pragma("unroll") for (int i = 0; i < KP; ++i) {                                                 \
+        const int idx = i * 256 + tid;                                                                 \
+        const int key = idx / CHUNKS, chunk = idx - key * CHUNKS;                                      \
+        const int j = ((KB) + key < kv_last) ? (KB) + key : kv_last;                                   \
+        int phys;                                                                                      \
+        AP_SLOT(j, phys);                                                                              \
+        kreg[i] = *reinterpret_cast<const u32x4*>(k_head + static_cast<size_t>(phys) * row_elems + chunk * 8); \
+      }                                                                                                \
+      _Pragma("unroll") for (int i = 0; i < VC; ++i) {                                                 \
+        const int idx = i * 256 + tid;                                                                 \
+        const int chunk = idx >> 4, quad = idx & 15;                                                   \
+        if (chunk < CHUNKS) {                                                                          \
+          _Pragma("unroll") for (int p = 0; p < 4; ++p) {                                              \
+            const int j = ((KB) + 4 * quad + p < kv_last) ? (KB) + 4 * quad + p : kv_last;             \
+            int phys;                                                                                  \
+            AP_SLOT(j, phys);                                                                          \
+            vreg[i][p] = *reinterpret_cast<const u32x4*>(v_head + static_cast<size_t>(phys) * row_elems + chunk * 8); \
+          }                                                                                            \
         }                                                                                              \
       }                                                                                                \
     }                                                                                                  \
@@ -321,16 +347,18 @@ extern "C" int pylon_attention_prefill(void* out, const void* q, const void* k_c
   const int group = n_heads / n_kv_heads;
   dim3 grid((n_tiles + per_wg - 1) / per_wg, n_kv_heads), block(256);
   const bool pow2 = (page_size & (page_size - 1)) == 0;
+  const int paging = !pow2 ? 0 : (page_size >= AP_BK ? 2 : 1);
+  PYLON_REQUIRE(static_cast<long long>(n_kv_heads) * head_dim * AP_BK < (1LL << 31),
+                "attention_prefill: %d key/value heads of %d elements are too wide", n_kv_heads, head_dim);
+#define GO_PAGING(HD, QT, PG)                                                                            \
+  hipLaunchKernelGGL((attention_prefill_kernel<HD, QT, PG>), grid, block, 0, stream, (uint16_t*)out,     \
+                     (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_table, \
+                     table_width, tiles, n_tiles, per_wg, n_heads, n_kv_heads, group, page_size, window, scale)
 #define GO(HD, QT)                                                                                       \
   do {                                                                                                   \
-    if (pow2)                                                                                            \
-      hipLaunchKernelGGL((attention_prefill_kernel<HD, QT, true>), grid, block, 0, stream, (uint16_t*)out, \
-                         (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache,         \
-                         block_table, table_width, tiles, n_tiles, per_wg, n_heads, n_kv_heads, group, page_size, window, scale); \
-    else                                                                                                 \
-      hipLaunchKernelGGL((attention_prefill_kernel<HD, QT, false>), grid, block, 0, stream, (uint16_t*)out, \
-                         (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache,         \
-                         block_table, table_width, tiles, n_tiles, per_wg, n_heads, n_kv_heads, group, page_size, window, scale); \
+    if (paging == 2) GO_PAGING(HD, QT, 2);                                                               \
+    else if (paging == 1) GO_PAGING(HD, QT, 1);                                                          \
+    else GO_PAGING(HD, QT, 0);                                                                           \
   } while (0)
   if (rows == 64) {
     if (head_dim == 64) GO(64, 1);
@@ -342,5 +370,6 @@ extern "C" int pylon_attention_prefill(void* out, const void* q, const void* k_c
     else GO(256, 2);
   }
 #undef GO
+#undef GO_PAGING
   PYLON_LAUNCHED("attention_prefill");
 }
