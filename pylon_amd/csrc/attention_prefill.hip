@@ -33,6 +33,123 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{lo, hi}, bf16x2));
 }
 
+// The queries of a wave: column `col` of query tile qt is (token, head) pair
+// wave*16*QT + qt*16 + col of the workgroup's tile; its position (or -1 if the tile has no
+// such pair) and its elements as column operands of the score product.
+template <int HD, int QT>
+__device__ __forceinline__ void load_queries(int (&qpos)[QT], bf16x8 (&qf)[QT][HD / 32], const uint16_t* __restrict__ q,
+                                             int wave, int col, int grp, int group, int tok0, int ntok, int pos0,
+                                             int n_heads, int head0) {
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    const int rr = wave * (16 * QT) + qt * 16 + col;
+    const int ti = rr / group, hh = rr - ti * group;
+    const bool valid = ti < ntok;
+    qpos[qt] = valid ? pos0 + ti : -1;
+    const uint16_t* qrow = q + (static_cast<size_t>(tok0 + (valid ? ti : 0)) * n_heads + head0 + hh) * HD;
+#pragma unroll
+    for (int ks = 0; ks < HD / 32; ++ks) {
+      if (valid) {
+        qf[qt][ks] = *reinterpret_cast<const bf16x8*>(qrow + ks * 32 + grp * 8);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) qf[qt][ks][i] = (__bf16)0.0f;
+      }
+    }
+  }
+}
+
+// One block of 64 keys for one query tile of a wave: s holds the transposed scores (lane
+// (col, grp) has keys kb + 16*kt + 4*grp + r of query column col).  Masks, keeps the
+// running maximum and sum, rescales the accumulators when the maximum moves, and returns
+// the probabilities as row operands of the value product: operand slot j of a lane is key
+// 32*kg + 4*grp + j (j < 4) or 32*kg + 16 + 4*grp + (j - 4).
+template <int DT>
+__device__ __forceinline__ void softmax_block(floatx4 (&s)[AP_BK / 16], bf16x8 (&pa)[AP_BK / 32], float& m_run,
+                                              float& l_run, floatx4 (&o)[DT], int qp, int kb, bool masked,
+                                              int window, int grp, float scale_log2, float slack) {
+  if (masked) {
+    const int lo = (window > 0) ? qp - window + 1 : 0;
+#pragma unroll
+    for (int kt = 0; kt < AP_BK / 16; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int key = kb + kt * 16 + 4 * grp + r;
+        if (!(key <= qp && key >= lo)) s[kt][r] = -INFINITY;
+      }
+  } else if (qp < 0) {  // a column that holds no query
+#pragma unroll
+    for (int kt = 0; kt < AP_BK / 16; ++kt) s[kt] = floatx4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+  }
+  // The maximum that the exponentials are taken against is raised only when a score
+  // exceeds it by more than AP_SLACK (in units of exp2's argument): until then
+  // probabilities may reach 2^AP_SLACK instead of 1, which float sums and bfloat16
+  // operands hold just as well, and neither the cross-lane maximum nor the rescaling
+  // of the accumulators is needed.  The result is the same up to rounding.
+  float tile_max = -INFINITY;
+#pragma unroll
+  for (int kt = 0; kt < AP_BK / 16; ++kt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) tile_max = fmaxf(tile_max, s[kt][r]);
+  if (__ballot(tile_max > m_run + slack) != 0) {  // the same for the whole wave
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, PYLON_WAVE));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, PYLON_WAVE));
+    const float m_new = fmaxf(m_run, tile_max);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen no key yet
+    const float corr = __builtin_amdgcn_exp2f((m_run - m_use) * scale_log2);
+    l_run *= corr;
+    m_run = m_new;
+    // the accumulators of this lane belong to query rows 4*grp + r: fetch their factors
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float c = __shfl(corr, 4 * grp + r, PYLON_WAVE);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[dt][r] *= c;
+    }
+  }
+  const float shift = (m_run == -INFINITY) ? 0.f : -m_run * scale_log2;
+  float p[AP_BK / 16][4];
+#pragma unroll
+  for (int kt = 0; kt < AP_BK / 16; ++kt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      p[kt][r] = __builtin_amdgcn_exp2f(fmaf(s[kt][r], scale_log2, shift));
+      l_run += p[kt][r];  // this lane's share of the row's sum; the lanes meet at the end
+    }
+#pragma unroll
+  for (int kg = 0; kg < AP_BK / 32; ++kg) {
+    const u32x4 packed = {pack_bf16(p[2 * kg][0], p[2 * kg][1]), pack_bf16(p[2 * kg][2], p[2 * kg][3]),
+                          pack_bf16(p[2 * kg + 1][0], p[2 * kg + 1][1]),
+                          pack_bf16(p[2 * kg + 1][2], p[2 * kg + 1][3])};
+    pa[kg] = __builtin_bit_cast(bf16x8, packed);
+  }
+}
+
+// out = acc / sum for a wave's query tiles; a lane holds rows 4*grp + r, element dt*16 + col.
+template <int HD, int QT>
+__device__ __forceinline__ void store_tile(uint16_t* __restrict__ out, const floatx4 (&o)[QT][HD / 16],
+                                           const float (&l_run)[QT], int wave, int col, int grp, int group,
+                                           int tok0, int ntok, int n_heads, int head0) {
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    float l_row = l_run[qt];  // the four lanes of a query column each hold a share
+    l_row += __shfl_xor(l_row, 16, PYLON_WAVE);
+    l_row += __shfl_xor(l_row, 32, PYLON_WAVE);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float l = __shfl(l_row, 4 * grp + r, PYLON_WAVE);
+      const int rr = wave * (16 * QT) + qt * 16 + 4 * grp + r;
+      const int ti = rr / group, hh = rr - ti * group;
+      if (ti < ntok) {
+        const float inv = 1.0f / l;
+        uint16_t* orow = out + (static_cast<size_t>(tok0 + ti) * n_heads + head0 + hh) * HD;
+#pragma unroll
+        for (int dt = 0; dt < HD / 16; ++dt) orow[dt * 16 + col] = float_to_bf16_bits(o[qt][dt][r] * inv);
+      }
+    }
+  }
+}
+
 // QT: 16-row query tiles per wave (1: 64 rows per workgroup, 2: 128).  PAGING says how a
 // key's place in the cache is found: 0 by a division by the page size (some twenty
 // instructions, eight times per thread and block), 1 by a shift and a mask (the page size is
@@ -139,26 +256,9 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
 
   AP_FETCH(kb_first);
 
-  // this lane's query column in each of the wave's query tiles
   int qpos[QT];
   bf16x8 qf[QT][KS];
-#pragma unroll
-  for (int qt = 0; qt < QT; ++qt) {
-    const int rr = wave * (16 * QT) + qt * 16 + col;
-    const int ti = rr / group, hh = rr - ti * group;
-    const bool valid = ti < ntok;
-    qpos[qt] = valid ? pos0 + ti : -1;
-    const uint16_t* qrow = q + (static_cast<size_t>(tok0 + (valid ? ti : 0)) * n_heads + kvh * group + hh) * HD;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      if (valid) {
-        qf[qt][ks] = *reinterpret_cast<const bf16x8*>(qrow + ks * 32 + grp * 8);
-      } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) qf[qt][ks][i] = (__bf16)0.0f;
-      }
-    }
-  }
+  load_queries<HD, QT>(qpos, qf, q, wave, col, grp, group, tok0, ntok, pos0, n_heads, kvh * group);
 
   float m_run[QT], l_run[QT];  // the running maximum is kept in units of raw scores
   floatx4 o[QT][DT];
@@ -219,67 +319,10 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     const bool masked = kb + AP_BK - 1 > pos0 || window > 0;
     bf16x8 pa[QT][AP_BK / 32];
 #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-      if (masked) {
-        const int qp = qpos[qt];
-        const int lo = (window > 0) ? qp - window + 1 : 0;
-#pragma unroll
-        for (int kt = 0; kt < AP_BK / 16; ++kt)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int key = kb + kt * 16 + 4 * grp + r;
-            if (!(key <= qp && key >= lo)) s[qt][kt][r] = -INFINITY;
-          }
-      } else if (qpos[qt] < 0) {  // a column that holds no query
-#pragma unroll
-        for (int kt = 0; kt < AP_BK / 16; ++kt) s[qt][kt] = floatx4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-      }
-      // The maximum that the exponentials are taken against is raised only when a score
-      // exceeds it by more than AP_SLACK (in units of exp2's argument): until then
-      // probabilities may reach 2^AP_SLACK instead of 1, which float sums and bfloat16
-      // operands hold just as well, and neither the cross-lane maximum nor the rescaling
-      // of the accumulators is needed.  The result is the same up to rounding.
-      float tile_max = -INFINITY;
-#pragma unroll
-      for (int kt = 0; kt < AP_BK / 16; ++kt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) tile_max = fmaxf(tile_max, s[qt][kt][r]);
-      if (__ballot(tile_max > m_run[qt] + slack) != 0) {  // the same for the whole wave
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, PYLON_WAVE));
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, PYLON_WAVE));
-        const float m_new = fmaxf(m_run[qt], tile_max);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen no key yet
-        const float corr = __builtin_amdgcn_exp2f((m_run[qt] - m_use) * scale_log2);
-        l_run[qt] *= corr;
-        m_run[qt] = m_new;
-        // the accumulators of this lane belong to query rows 4*grp + r: fetch their factors
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float c = __shfl(corr, 4 * grp + r, PYLON_WAVE);
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) o[qt][dt][r] *= c;
-        }
-      }
-      const float shift = (m_run[qt] == -INFINITY) ? 0.f : -m_run[qt] * scale_log2;
-      float p[AP_BK / 16][4];
-#pragma unroll
-      for (int kt = 0; kt < AP_BK / 16; ++kt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          p[kt][r] = __builtin_amdgcn_exp2f(fmaf(s[qt][kt][r], scale_log2, shift));
-          l_run[qt] += p[kt][r];  // this lane's share of the row's sum; the lanes meet at the end
-        }
-#pragma unroll
-      for (int kg = 0; kg < AP_BK / 32; ++kg) {
-        const u32x4 packed = {pack_bf16(p[2 * kg][0], p[2 * kg][1]), pack_bf16(p[2 * kg][2], p[2 * kg][3]),
-                              pack_bf16(p[2 * kg + 1][0], p[2 * kg + 1][1]),
-                              pack_bf16(p[2 * kg + 1][2], p[2 * kg + 1][3])};
-        pa[qt][kg] = __builtin_bit_cast(bf16x8, packed);
-      }
-    }
+    for (int qt = 0; qt < QT; ++qt)
+      softmax_block<DT>(s[qt], pa[qt], m_run[qt], l_run[qt], o[qt], qpos[qt], kb, masked, window, grp, scale_log2, slack);
 
-    // out += P * V; operand slot j of a lane is key 32*kg + 4*grp + j (j < 4) or
-    // 32*kg + 16 + 4*grp + (j - 4), for P and V alike
+    // out += P * V, the values in the same order of keys as the probabilities
 #pragma unroll
     for (int kg = 0; kg < AP_BK / 32; ++kg) {
 #pragma unroll
@@ -298,26 +341,166 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
 #undef AP_FETCH
 #undef AP_SLOT
 
-  // out = acc / sum; this lane holds rows 4*grp + r, element dt*16 + col
+  store_tile<HD, QT>(out, o, l_run, wave, col, grp, group, tok0, ntok, n_heads, kvh * group);
+  __syncthreads();  // LDS (the page table, the last block) is free for the next tile
+  }
+}
+
+// The same for head size 128 and pages that are powers of two of at least 64, with the two
+// matrix-instruction-era features of this chip that take the copying out of the loop:
+//
+//  * Keys and values go from the cache straight into LDS (16 bytes per lane, a wave fills
+//    1 KB of consecutive LDS from 64 places of its choice), two buffers each, so that the
+//    next block travels while this one is used, with one barrier per block and no staging
+//    registers.  A row of a tile is 256 bytes without padding; bank conflicts are avoided
+//    by a swizzle on the way in: the 16-byte piece c of key row r lies at piece c ^ (r % 16)
+//    (keys) or c ^ (2 * (r % 8)) (values).
+//  * The values stay row-major: the transposing LDS read hands a lane, for its column of
+//    the output tile, the elements of four consecutive keys, which is the column operand of
+//    the value product (lane p of a group of 16 names row p / 4, elements 4 * (p % 4) .. + 3;
+//    lane i receives element i % 4 of lanes i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12).
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+#define AP_LDS(T) __attribute__((address_space(3))) T
+#define AP_GLOBAL(T) __attribute__((address_space(1))) T
+
+template <int QT>
+__global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
+    uint16_t* __restrict__ out, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
+    const uint16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
+    const int* __restrict__ tiles, int n_tiles, int per_wg, int n_heads, int n_kv_heads, int group,
+    int page_size, int window, float scale) {
+  constexpr int HD = 128, KS = HD / 32, DT = HD / 16;
+  constexpr int ROW = HD * 2;  // bytes of a key or value row in LDS
+  __shared__ __attribute__((aligned(16))) uint16_t k_a[AP_BK * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t k_b[AP_BK * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t v_a[AP_BK * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t v_b[AP_BK * HD];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 15, grp = lane >> 4;
+  const int kvh = blockIdx.y;
+  const int page_shift = __ffs(page_size) - 1, page_mask = page_size - 1;
+  const size_t row_elems = static_cast<size_t>(n_kv_heads) * HD;
+  const unsigned row_elems32 = n_kv_heads * HD;
+  const uint16_t* k_head = k_cache + static_cast<size_t>(kvh) * HD;
+  const uint16_t* v_head = v_cache + static_cast<size_t>(kvh) * HD;
+
+  // Where this lane reads its operands (bytes from a tile's start).  Keys: row col of a
+  // 16-key tile, piece ks*4 + grp.  Values: row 4*grp + col/4 of a 32-key group, the 8 bytes
+  // at element dt*16 + 4*(col%4).
+  unsigned k_at[KS], v_at[DT];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) k_at[ks] = col * ROW + (((ks * 4 + grp) ^ col) * 16);
+  {
+    const unsigned vrow = 4 * grp + (col >> 2), swizzle = 2 * (vrow & 7);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      v_at[dt] = vrow * ROW + (((2 * dt + ((col & 3) >> 1)) ^ swizzle) * 16) + (col & 1) * 8;
+  }
+  // What this lane brings in: load i of its wave fills rows 16*wave + 4*i + grp, piece col.
+  unsigned k_piece[4], v_piece[4];  // element offsets inside the cache row, swizzle applied
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const unsigned r = 4 * i + grp;
+    k_piece[i] = (col ^ r) * 8;
+    v_piece[i] = (col ^ (2 * (r & 7))) * 8;
+  }
+
+  for (int part = 0; part < per_wg; ++part) {
+  const int tile = blockIdx.x * per_wg + part;
+  if (tile >= n_tiles) break;
+  const int* td = tiles + tile * 4;
+  const int tok0 = td[0], ntok = td[1], trow = td[2], pos0 = td[3];
+  const int* table = block_table + static_cast<size_t>(trow) * table_width;
+  const int kv_last = pos0 + ntok - 1;
+  const int k_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int kb_first = (k_lo / AP_BK) * AP_BK;
+
+  // A block of 64 keys lies inside one page.  Rows past the last key repeat it.
+#define APD_FETCH(KB, KBUF, VBUF)                                                                      \
+  do {                                                                                                 \
+    const int page_row = table[(KB) >> page_shift] * page_size + ((KB) & page_mask);                   \
+    const uint16_t* k_block = k_head + static_cast<size_t>(page_row) * row_elems;                      \
+    const uint16_t* v_block = v_head + static_cast<size_t>(page_row) * row_elems;                      \
+    const unsigned last = kv_last - (KB);                                                              \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                    \
+      const unsigned r = 16 * wave + 4 * i + grp;                                                      \
+      const unsigned row = (r < last ? r : last) * row_elems32;                                        \
+      __builtin_amdgcn_global_load_lds((const AP_GLOBAL(void)*)(k_block + (row + k_piece[i])),         \
+                                       (AP_LDS(void)*)((KBUF) + (16 * wave + 4 * i) * HD), 16, 0, 0);  \
+      __builtin_amdgcn_global_load_lds((const AP_GLOBAL(void)*)(v_block + (row + v_piece[i])),         \
+                                       (AP_LDS(void)*)((VBUF) + (16 * wave + 4 * i) * HD), 16, 0, 0);  \
+    }                                                                                                  \
+  } while (0)
+
+  APD_FETCH(kb_first, k_a, v_a);
+
+  int qpos[QT];
+  bf16x8 qf[QT][KS];
+  load_queries<HD, QT>(qpos, qf, q, wave, col, grp, group, tok0, ntok, pos0, n_heads, kvh * group);
+
+  float m_run[QT], l_run[QT];  // the running maximum is kept in units of raw scores
+  floatx4 o[QT][DT];
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
-    float l_row = l_run[qt];  // the four lanes of a query column each hold a share
-    l_row += __shfl_xor(l_row, 16, PYLON_WAVE);
-    l_row += __shfl_xor(l_row, 32, PYLON_WAVE);
+    m_run[qt] = -INFINITY;
+    l_run[qt] = 0.f;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float l = __shfl(l_row, 4 * grp + r, PYLON_WAVE);
-      const int rr = wave * (16 * QT) + qt * 16 + 4 * grp + r;
-      const int ti = rr / group, hh = rr - ti * group;
-      if (ti < ntok) {
-        const float inv = 1.0f / l;
-        uint16_t* orow = out + (static_cast<size_t>(tok0 + ti) * n_heads + kvh * group + hh) * HD;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) orow[dt * 16 + col] = float_to_bf16_bits(o[qt][dt][r] * inv);
-      }
-    }
+    for (int dt = 0; dt < DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
-  __syncthreads();  // LDS (the page table, the last block) is free for the next tile
+  const float scale_log2 = scale * 1.44269504088896340736f;
+  const float slack = AP_SLACK / scale_log2;  // in units of raw scores
+
+  // One block: wait for its keys and values (this wave's loads, then everyone's), send for
+  // the next block into the other buffers (their last readers are past the barrier), and
+  // do the math from LDS.
+#define APD_BLOCK(KB, KCUR, VCUR, KNEXT, VNEXT)                                                        \
+  do {                                                                                                 \
+    __builtin_amdgcn_s_waitcnt(0);                                                                     \
+    __syncthreads();                                                                                   \
+    if ((KB) + AP_BK <= kv_last) APD_FETCH((KB) + AP_BK, KNEXT, VNEXT);                                \
+    const AP_LDS(char)* k_tile = (const AP_LDS(char)*)(KCUR);                                          \
+    const AP_LDS(char)* v_tile = (const AP_LDS(char)*)(VCUR);                                          \
+    floatx4 s[QT][AP_BK / 16];                                                                         \
+    _Pragma("unroll") for (int kt = 0; kt < AP_BK / 16; ++kt) {                                        \
+      _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                              \
+        const bf16x8 kf = *reinterpret_cast<const AP_LDS(bf16x8)*>(k_tile + k_at[ks] + kt * 16 * ROW); \
+        _Pragma("unroll") for (int qt = 0; qt < QT; ++qt)                                              \
+          s[qt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(                                         \
+              kf, qf[qt][ks], ks == 0 ? floatx4{0.f, 0.f, 0.f, 0.f} : s[qt][kt], 0, 0, 0);             \
+      }                                                                                                \
+    }                                                                                                  \
+    const bool masked = (KB) + AP_BK - 1 > pos0 || window > 0;                                         \
+    bf16x8 pa[QT][AP_BK / 32];                                                                         \
+    _Pragma("unroll") for (int qt = 0; qt < QT; ++qt)                                                  \
+      softmax_block<DT>(s[qt], pa[qt], m_run[qt], l_run[qt], o[qt], qpos[qt], (KB), masked, window,    \
+                        grp, scale_log2, slack);                                                       \
+    _Pragma("unroll") for (int kg = 0; kg < AP_BK / 32; ++kg) {                                        \
+      _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                              \
+        const s16x4 first = __builtin_amdgcn_ds_read_tr16_b64_v4i16(                                   \
+            (AP_LDS(s16x4)*)(v_tile + v_at[dt] + kg * 32 * ROW));                                      \
+        const s16x4 second = __builtin_amdgcn_ds_read_tr16_b64_v4i16(                                  \
+            (AP_LDS(s16x4)*)(v_tile + v_at[dt] + kg * 32 * ROW + 16 * ROW));                           \
+        const bf16x8 vf = __builtin_bit_cast(                                                          \
+            bf16x8, __builtin_shufflevector(first, second, 0, 1, 2, 3, 4, 5, 6, 7));                   \
+        _Pragma("unroll") for (int qt = 0; qt < QT; ++qt)                                              \
+          o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[qt][kg], vf, o[qt][dt], 0, 0, 0);     \
+      }                                                                                                \
+    }                                                                                                  \
+  } while (0)
+
+  for (int kb = kb_first;; kb += 2 * AP_BK) {
+    APD_BLOCK(kb, k_a, v_a, k_b, v_b);
+    if (kb + AP_BK > kv_last) break;
+    APD_BLOCK(kb + AP_BK, k_b, v_b, k_a, v_a);
+    if (kb + 2 * AP_BK > kv_last) break;
+  }
+#undef APD_BLOCK
+#undef APD_FETCH
+
+  store_tile<HD, QT>(out, o, l_run, wave, col, grp, group, tok0, ntok, n_heads, kvh * group);
+  __syncthreads();  // the buffers are free for the next tile
   }
 }
 
@@ -360,7 +543,14 @@ extern "C" int pylon_attention_prefill(void* out, const void* q, const void* k_c
     else if (paging == 1) GO_PAGING(HD, QT, 1);                                                          \
     else GO_PAGING(HD, QT, 0);                                                                           \
   } while (0)
-  if (rows == 64) {
+  if (head_dim == 128 && paging == 2) {
+#define GO_DIRECT(QT)                                                                                    \
+  hipLaunchKernelGGL((attention_prefill_direct_kernel<QT>), grid, block, 0, stream, (uint16_t*)out,      \
+                     (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_table, \
+                     table_width, tiles, n_tiles, per_wg, n_heads, n_kv_heads, group, page_size, window, scale)
+    if (rows == 64) GO_DIRECT(1); else GO_DIRECT(2);
+#undef GO_DIRECT
+  } else if (rows == 64) {
     if (head_dim == 64) GO(64, 1);
     else if (head_dim == 128) GO(128, 1);
     else GO(256, 1);
