@@ -61,22 +61,26 @@ __device__ __forceinline__ void load_queries(int (&qpos)[QT], bf16x8 (&qf)[QT][H
 
 // One block of 64 keys for one query tile of a wave: s holds the transposed scores (lane
 // (col, grp) has keys kb + 16*kt + 4*grp + r of query column col).  Masks, keeps the
-// running maximum and sum, rescales the accumulators when the maximum moves, and returns
+// running maximum, rescales the NT accumulator tiles when the maximum moves, and returns
 // the probabilities as row operands of the value product: operand slot j of a lane is key
-// 32*kg + 4*grp + j (j < 4) or 32*kg + 16 + 4*grp + (j - 4).
-template <int DT>
+// 32*kg + 4*grp + j (j < 4) or 32*kg + 16 + 4*grp + (j - 4).  The row sums are not kept
+// here: the caller multiplies the probabilities by a tile of ones as well, so that the last
+// accumulator tile holds, in every column, the sum of exactly the rounded probabilities that
+// weigh the values.
+template <int NT>
 __device__ __forceinline__ void softmax_block(floatx4 (&s)[AP_BK / 16], bf16x8 (&pa)[AP_BK / 32], float& m_run,
-                                              float& l_run, floatx4 (&o)[DT], int qp, int kb, bool masked,
-                                              int window, int grp, float scale_log2, float slack) {
+                                              floatx4 (&o)[NT], int qp, int kb, bool masked, int window, int grp,
+                                              float scale_log2, float slack) {
   if (masked) {
-    const int lo = (window > 0) ? qp - window + 1 : 0;
+    // key kb + 16*kt + 4*grp + r is seen if it is at most qp and inside the window: compared
+    // as 16*kt + r (a constant) against two numbers of this lane
+    const int last_seen = qp - kb - 4 * grp;
+    const int first_seen = (window > 0) ? last_seen - window + 1 : -(1 << 30);
 #pragma unroll
     for (int kt = 0; kt < AP_BK / 16; ++kt)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int key = kb + kt * 16 + 4 * grp + r;
-        if (!(key <= qp && key >= lo)) s[kt][r] = -INFINITY;
-      }
+      for (int r = 0; r < 4; ++r)
+        if (!(kt * 16 + r <= last_seen && kt * 16 + r >= first_seen)) s[kt][r] = -INFINITY;
   } else if (qp < 0) {  // a column that holds no query
 #pragma unroll
     for (int kt = 0; kt < AP_BK / 16; ++kt) s[kt] = floatx4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
@@ -97,14 +101,13 @@ __device__ __forceinline__ void softmax_block(floatx4 (&s)[AP_BK / 16], bf16x8 (
     const float m_new = fmaxf(m_run, tile_max);
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a row that has seen no key yet
     const float corr = __builtin_amdgcn_exp2f((m_run - m_use) * scale_log2);
-    l_run *= corr;
     m_run = m_new;
     // the accumulators of this lane belong to query rows 4*grp + r: fetch their factors
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const float c = __shfl(corr, 4 * grp + r, PYLON_WAVE);
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) o[dt][r] *= c;
+      for (int nt = 0; nt < NT; ++nt) o[nt][r] *= c;
     }
   }
   const float shift = (m_run == -INFINITY) ? 0.f : -m_run * scale_log2;
@@ -112,10 +115,7 @@ __device__ __forceinline__ void softmax_block(floatx4 (&s)[AP_BK / 16], bf16x8 (
 #pragma unroll
   for (int kt = 0; kt < AP_BK / 16; ++kt)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      p[kt][r] = __builtin_amdgcn_exp2f(fmaf(s[kt][r], scale_log2, shift));
-      l_run += p[kt][r];  // this lane's share of the row's sum; the lanes meet at the end
-    }
+    for (int r = 0; r < 4; ++r) p[kt][r] = __builtin_amdgcn_exp2f(fmaf(s[kt][r], scale_log2, shift));
 #pragma unroll
   for (int kg = 0; kg < AP_BK / 32; ++kg) {
     const u32x4 packed = {pack_bf16(p[2 * kg][0], p[2 * kg][1]), pack_bf16(p[2 * kg][2], p[2 * kg][3]),
@@ -125,19 +125,17 @@ __device__ __forceinline__ void softmax_block(floatx4 (&s)[AP_BK / 16], bf16x8 (
   }
 }
 
-// out = acc / sum for a wave's query tiles; a lane holds rows 4*grp + r, element dt*16 + col.
+// out = acc / sum for a wave's query tiles; a lane holds rows 4*grp + r, element dt*16 + col,
+// and the rows' sums in the tile after the last.
 template <int HD, int QT>
-__device__ __forceinline__ void store_tile(uint16_t* __restrict__ out, const floatx4 (&o)[QT][HD / 16],
-                                           const float (&l_run)[QT], int wave, int col, int grp, int group,
-                                           int tok0, int ntok, int n_heads, int head0) {
+__device__ __forceinline__ void store_tile(uint16_t* __restrict__ out, const floatx4 (&o)[QT][HD / 16 + 1], int wave,
+                                           int col, int grp, int group, int tok0, int ntok, int n_heads,
+                                           int head0) {
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
-    float l_row = l_run[qt];  // the four lanes of a query column each hold a share
-    l_row += __shfl_xor(l_row, 16, PYLON_WAVE);
-    l_row += __shfl_xor(l_row, 32, PYLON_WAVE);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const float l = __shfl(l_row, 4 * grp + r, PYLON_WAVE);
+      const float l = o[qt][HD / 16][r];
       const int rr = wave * (16 * QT) + qt * 16 + 4 * grp + r;
       const int ti = rr / group, hh = rr - ti * group;
       if (ti < ntok) {
@@ -174,11 +172,14 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, grp = lane >> 4;
-  const int kvh = blockIdx.y;
+  // Workgroups start in the order of blockIdx.x and go round the chip's eight dies, each with
+  // a cache of its own: neighbours take the same tile for different key/value heads, so the
+  // heaviest tiles of all heads start first and a die meets few heads.
+  const int kvh = blockIdx.x % n_kv_heads, slot = blockIdx.x / n_kv_heads;
   // A workgroup takes per_wg tiles one after the other (the host pairs a long one with a
   // short one, so that every workgroup has about the same number of key blocks to walk).
   for (int part = 0; part < per_wg; ++part) {
-  const int tile = blockIdx.x * per_wg + part;
+  const int tile = slot * per_wg + part;
   if (tile >= n_tiles) break;
   const int* td = tiles + tile * 4;
   const int tok0 = td[0], ntok = td[1], trow = td[2], pos0 = td[3];
@@ -260,15 +261,15 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   bf16x8 qf[QT][KS];
   load_queries<HD, QT>(qpos, qf, q, wave, col, grp, group, tok0, ntok, pos0, n_heads, kvh * group);
 
-  float m_run[QT], l_run[QT];  // the running maximum is kept in units of raw scores
-  floatx4 o[QT][DT];
+  float m_run[QT];          // the running maximum, in units of raw scores
+  floatx4 o[QT][DT + 1];    // the output tiles and, last, the rows' sums
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     m_run[qt] = -INFINITY;
-    l_run[qt] = 0.f;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int dt = 0; dt <= DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
+  const bf16x8 ones = __builtin_bit_cast(bf16x8, u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u});
 
   const float scale_log2 = scale * 1.44269504088896340736f;
   const float slack = AP_SLACK / scale_log2;  // in units of raw scores
@@ -320,7 +321,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     bf16x8 pa[QT][AP_BK / 32];
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt)
-      softmax_block<DT>(s[qt], pa[qt], m_run[qt], l_run[qt], o[qt], qpos[qt], kb, masked, window, grp, scale_log2, slack);
+      softmax_block<DT + 1>(s[qt], pa[qt], m_run[qt], o[qt], qpos[qt], kb, masked, window, grp, scale_log2, slack);
 
     // out += P * V, the values in the same order of keys as the probabilities
 #pragma unroll
@@ -336,12 +337,15 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
         for (int qt = 0; qt < QT; ++qt)
           o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[qt][kg], vf, o[qt][dt], 0, 0, 0);
       }
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt)
+        o[qt][DT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[qt][kg], ones, o[qt][DT], 0, 0, 0);
     }
   }
 #undef AP_FETCH
 #undef AP_SLOT
 
-  store_tile<HD, QT>(out, o, l_run, wave, col, grp, group, tok0, ntok, n_heads, kvh * group);
+  store_tile<HD, QT>(out, o, wave, col, grp, group, tok0, ntok, n_heads, kvh * group);
   __syncthreads();  // LDS (the page table, the last block) is free for the next tile
   }
 }
@@ -360,6 +364,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
 //    the value product (lane p of a group of 16 names row p / 4, elements 4 * (p % 4) .. + 3;
 //    lane i receives element i % 4 of lanes i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12).
 typedef short s16x4 __attribute__((ext_vector_type(4)));
+#define AP_VAHEAD 4  // value operands (16-element output tiles) read ahead of their products
 #define AP_LDS(T) __attribute__((address_space(3))) T
 #define AP_GLOBAL(T) __attribute__((address_space(1))) T
 
@@ -379,7 +384,10 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, grp = lane >> 4;
-  const int kvh = blockIdx.y;
+  // Workgroups start in the order of blockIdx.x and go round the chip's eight dies, each with
+  // a cache of its own: neighbours take the same tile for different key/value heads, so the
+  // heaviest tiles of all heads start first and a die meets few heads.
+  const int kvh = blockIdx.x % n_kv_heads, slot = blockIdx.x / n_kv_heads;
   const int page_shift = __ffs(page_size) - 1, page_mask = page_size - 1;
   const size_t row_elems = static_cast<size_t>(n_kv_heads) * HD;
   const unsigned row_elems32 = n_kv_heads * HD;
@@ -408,7 +416,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
   }
 
   for (int part = 0; part < per_wg; ++part) {
-  const int tile = blockIdx.x * per_wg + part;
+  const int tile = slot * per_wg + part;
   if (tile >= n_tiles) break;
   const int* td = tiles + tile * 4;
   const int tok0 = td[0], ntok = td[1], trow = td[2], pos0 = td[3];
@@ -440,15 +448,15 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
   bf16x8 qf[QT][KS];
   load_queries<HD, QT>(qpos, qf, q, wave, col, grp, group, tok0, ntok, pos0, n_heads, kvh * group);
 
-  float m_run[QT], l_run[QT];  // the running maximum is kept in units of raw scores
-  floatx4 o[QT][DT];
+  float m_run[QT];          // the running maximum, in units of raw scores
+  floatx4 o[QT][DT + 1];    // the output tiles and, last, the rows' sums
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     m_run[qt] = -INFINITY;
-    l_run[qt] = 0.f;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int dt = 0; dt <= DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
+  const bf16x8 ones = __builtin_bit_cast(bf16x8, u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u});
   const float scale_log2 = scale * 1.44269504088896340736f;
   const float slack = AP_SLACK / scale_log2;  // in units of raw scores
 
@@ -462,32 +470,55 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
     if ((KB) + AP_BK <= kv_last) APD_FETCH((KB) + AP_BK, KNEXT, VNEXT);                                \
     const AP_LDS(char)* k_tile = (const AP_LDS(char)*)(KCUR);                                          \
     const AP_LDS(char)* v_tile = (const AP_LDS(char)*)(VCUR);                                          \
+    /* scores: the operands of the next 16 keys are read while this tile's products run */             \
     floatx4 s[QT][AP_BK / 16];                                                                         \
+    bf16x8 kf[2][KS];                                                                                  \
+    _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                                  \
+      kf[0][ks] = *reinterpret_cast<const AP_LDS(bf16x8)*>(k_tile + k_at[ks]);                         \
     _Pragma("unroll") for (int kt = 0; kt < AP_BK / 16; ++kt) {                                        \
-      _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                              \
-        const bf16x8 kf = *reinterpret_cast<const AP_LDS(bf16x8)*>(k_tile + k_at[ks] + kt * 16 * ROW); \
+      if (kt + 1 < AP_BK / 16) {                                                                       \
+        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                              \
+          kf[(kt + 1) & 1][ks] =                                                                       \
+              *reinterpret_cast<const AP_LDS(bf16x8)*>(k_tile + k_at[ks] + (kt + 1) * 16 * ROW);       \
+      }                                                                                                \
+      __builtin_amdgcn_sched_barrier(0);                                                               \
+      _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                                \
         _Pragma("unroll") for (int qt = 0; qt < QT; ++qt)                                              \
           s[qt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(                                         \
-              kf, qf[qt][ks], ks == 0 ? floatx4{0.f, 0.f, 0.f, 0.f} : s[qt][kt], 0, 0, 0);             \
-      }                                                                                                \
+              kf[kt & 1][ks], qf[qt][ks], ks == 0 ? floatx4{0.f, 0.f, 0.f, 0.f} : s[qt][kt], 0, 0, 0); \
+      __builtin_amdgcn_sched_barrier(0);                                                               \
     }                                                                                                  \
+    /* the first values are on their way from LDS during the softmax */                                \
+    s16x4 vf[AP_VAHEAD][2];                                                                            \
+    _Pragma("unroll") for (int a = 0; a < AP_VAHEAD; ++a) {                                            \
+      vf[a][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((AP_LDS(s16x4)*)(v_tile + v_at[a]));          \
+      vf[a][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((AP_LDS(s16x4)*)(v_tile + v_at[a] + 16 * ROW)); \
+    }                                                                                                  \
+    __builtin_amdgcn_sched_barrier(0);                                                                 \
     const bool masked = (KB) + AP_BK - 1 > pos0 || window > 0;                                         \
     bf16x8 pa[QT][AP_BK / 32];                                                                         \
     _Pragma("unroll") for (int qt = 0; qt < QT; ++qt)                                                  \
-      softmax_block<DT>(s[qt], pa[qt], m_run[qt], l_run[qt], o[qt], qpos[qt], (KB), masked, window,    \
-                        grp, scale_log2, slack);                                                       \
-    _Pragma("unroll") for (int kg = 0; kg < AP_BK / 32; ++kg) {                                        \
-      _Pragma("unroll") for (int dt = 0; dt < DT; ++dt) {                                              \
-        const s16x4 first = __builtin_amdgcn_ds_read_tr16_b64_v4i16(                                   \
-            (AP_LDS(s16x4)*)(v_tile + v_at[dt] + kg * 32 * ROW));                                      \
-        const s16x4 second = __builtin_amdgcn_ds_read_tr16_b64_v4i16(                                  \
-            (AP_LDS(s16x4)*)(v_tile + v_at[dt] + kg * 32 * ROW + 16 * ROW));                           \
-        const bf16x8 vf = __builtin_bit_cast(                                                          \
-            bf16x8, __builtin_shufflevector(first, second, 0, 1, 2, 3, 4, 5, 6, 7));                   \
-        _Pragma("unroll") for (int qt = 0; qt < QT; ++qt)                                              \
-          o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[qt][kg], vf, o[qt][dt], 0, 0, 0);     \
+      softmax_block<DT + 1>(s[qt], pa[qt], m_run[qt], o[qt], qpos[qt], (KB), masked, window, grp,      \
+                            scale_log2, slack);                                                        \
+    __builtin_amdgcn_sched_barrier(0);                                                                 \
+    _Pragma("unroll") for (int it = 0; it < 2 * DT; ++it) {  /* it = kg * DT + dt */                   \
+      const bf16x8 vnow = __builtin_bit_cast(                                                          \
+          bf16x8, __builtin_shufflevector(vf[it % AP_VAHEAD][0], vf[it % AP_VAHEAD][1], 0, 1, 2, 3, 4, 5, 6, 7)); \
+      if (it + AP_VAHEAD < 2 * DT) {                                                                   \
+        const int nkg = (it + AP_VAHEAD) / DT, ndt = (it + AP_VAHEAD) % DT;                            \
+        vf[it % AP_VAHEAD][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(                               \
+            (AP_LDS(s16x4)*)(v_tile + v_at[ndt] + nkg * 32 * ROW));                                    \
+        vf[it % AP_VAHEAD][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(                               \
+            (AP_LDS(s16x4)*)(v_tile + v_at[ndt] + nkg * 32 * ROW + 16 * ROW));                         \
       }                                                                                                \
+      __builtin_amdgcn_sched_barrier(0);                                                               \
+      _Pragma("unroll") for (int qt = 0; qt < QT; ++qt)                                                \
+        o[qt][it % DT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[qt][it / DT], vnow, o[qt][it % DT], 0, 0, 0); \
+      __builtin_amdgcn_sched_barrier(0);                                                               \
     }                                                                                                  \
+    _Pragma("unroll") for (int kg = 0; kg < AP_BK / 32; ++kg)                                          \
+      _Pragma("unroll") for (int qt = 0; qt < QT; ++qt)                                                \
+        o[qt][DT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[qt][kg], ones, o[qt][DT], 0, 0, 0);     \
   } while (0)
 
   for (int kb = kb_first;; kb += 2 * AP_BK) {
@@ -499,7 +530,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
 #undef APD_BLOCK
 #undef APD_FETCH
 
-  store_tile<HD, QT>(out, o, l_run, wave, col, grp, group, tok0, ntok, n_heads, kvh * group);
+  store_tile<HD, QT>(out, o, wave, col, grp, group, tok0, ntok, n_heads, kvh * group);
   __syncthreads();  // the buffers are free for the next tile
   }
 }
@@ -525,10 +556,10 @@ extern "C" int pylon_attention_prefill(void* out, const void* q, const void* k_c
   PYLON_REQUIRE(page_size > 0 && table_width > 0 && window >= 0, "attention_prefill: bad page size, width or window");
   PYLON_REQUIRE(table_width <= AP_TABLE, "attention_prefill: a request may hold at most %d pages, the table has %d columns",
                 AP_TABLE, table_width);
-  PYLON_REQUIRE(n_kv_heads <= 65535, "attention_prefill: too many key/value heads for one launch");
+  PYLON_REQUIRE(static_cast<long long>(n_tiles) * n_kv_heads < (1LL << 31), "attention_prefill: too many tiles for one launch");
   if (n_tiles == 0) return 0;
   const int group = n_heads / n_kv_heads;
-  dim3 grid((n_tiles + per_wg - 1) / per_wg, n_kv_heads), block(256);
+  dim3 grid(((n_tiles + per_wg - 1) / per_wg) * n_kv_heads), block(256);
   const bool pow2 = (page_size & (page_size - 1)) == 0;
   const int paging = !pow2 ? 0 : (page_size >= AP_BK ? 2 : 1);
   PYLON_REQUIRE(static_cast<long long>(n_kv_heads) * head_dim * AP_BK < (1LL << 31),
