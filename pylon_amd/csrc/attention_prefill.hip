@@ -157,7 +157,7 @@ template <int HD, int QT, int PAGING>
 __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
-    const int* __restrict__ tiles, int n_tiles, int per_wg, int n_heads, int n_kv_heads, int group,
+    const int* __restrict__ tiles, int n_heads, int n_kv_heads, int group,
     int page_size, int window, float scale) {
   constexpr int KS = HD / 32;        // 32-wide steps along the head for a score tile
   constexpr int DT = HD / 16;        // 16-wide output tiles along the head
@@ -175,12 +175,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   // Workgroups start in the order of blockIdx.x and go round the chip's eight dies, each with
   // a cache of its own: neighbours take the same tile for different key/value heads, so the
   // heaviest tiles of all heads start first and a die meets few heads.
-  const int kvh = blockIdx.x % n_kv_heads, slot = blockIdx.x / n_kv_heads;
-  // A workgroup takes per_wg tiles one after the other (the host pairs a long one with a
-  // short one, so that every workgroup has about the same number of key blocks to walk).
-  for (int part = 0; part < per_wg; ++part) {
-  const int tile = slot * per_wg + part;
-  if (tile >= n_tiles) break;
+  const int kvh = blockIdx.x % n_kv_heads, tile = blockIdx.x / n_kv_heads;
   const int* td = tiles + tile * 4;
   const int tok0 = td[0], ntok = td[1], trow = td[2], pos0 = td[3];
   const int* table = block_table + static_cast<size_t>(trow) * table_width;
@@ -346,8 +341,6 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
 #undef AP_SLOT
 
   store_tile<HD, QT>(out, o, wave, col, grp, group, tok0, ntok, n_heads, kvh * group);
-  __syncthreads();  // LDS (the page table, the last block) is free for the next tile
-  }
 }
 
 // The same for head size 128 and pages that are powers of two of at least 64, with the two
@@ -372,7 +365,7 @@ template <int QT>
 __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
-    const int* __restrict__ tiles, int n_tiles, int per_wg, int n_heads, int n_kv_heads, int group,
+    const int* __restrict__ tiles, int n_heads, int n_kv_heads, int group,
     int page_size, int window, float scale) {
   constexpr int HD = 128, KS = HD / 32, DT = HD / 16;
   constexpr int ROW = HD * 2;  // bytes of a key or value row in LDS
@@ -387,7 +380,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
   // Workgroups start in the order of blockIdx.x and go round the chip's eight dies, each with
   // a cache of its own: neighbours take the same tile for different key/value heads, so the
   // heaviest tiles of all heads start first and a die meets few heads.
-  const int kvh = blockIdx.x % n_kv_heads, slot = blockIdx.x / n_kv_heads;
+  const int kvh = blockIdx.x % n_kv_heads, tile = blockIdx.x / n_kv_heads;
   const int page_shift = __ffs(page_size) - 1, page_mask = page_size - 1;
   const size_t row_elems = static_cast<size_t>(n_kv_heads) * HD;
   const unsigned row_elems32 = n_kv_heads * HD;
@@ -415,9 +408,6 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
     v_piece[i] = (col ^ (2 * (r & 7))) * 8;
   }
 
-  for (int part = 0; part < per_wg; ++part) {
-  const int tile = slot * per_wg + part;
-  if (tile >= n_tiles) break;
   const int* td = tiles + tile * 4;
   const int tok0 = td[0], ntok = td[1], trow = td[2], pos0 = td[3];
   const int* table = block_table + static_cast<size_t>(trow) * table_width;
@@ -531,8 +521,6 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
 #undef APD_FETCH
 
   store_tile<HD, QT>(out, o, wave, col, grp, group, tok0, ntok, n_heads, kvh * group);
-  __syncthreads();  // the buffers are free for the next tile
-  }
 }
 
 // tiles: [n_tiles, 4] = (index of the tile's first token in q/out, its token count, its row of
@@ -542,9 +530,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
 extern "C" int pylon_attention_prefill(void* out, const void* q, const void* k_cache, const void* v_cache,
                                        const int* block_table, int table_width, const int* tiles,
                                        int n_tiles, int n_heads, int n_kv_heads, int head_dim,
-                                       int page_size, int window, float scale, int rows, int per_wg,
-                                       hipStream_t stream) {
-  PYLON_REQUIRE(per_wg >= 1 && per_wg <= 8, "attention_prefill: 1..8 tiles per workgroup, got %d", per_wg);
+                                       int page_size, int window, float scale, int rows, hipStream_t stream) {
   PYLON_REQUIRE(rows == 64 || rows == 128, "attention_prefill: 64 or 128 query rows per workgroup, got %d", rows);
   PYLON_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "attention_prefill: %d query heads cannot be grouped over %d key/value heads", n_heads,
@@ -559,7 +545,7 @@ extern "C" int pylon_attention_prefill(void* out, const void* q, const void* k_c
   PYLON_REQUIRE(static_cast<long long>(n_tiles) * n_kv_heads < (1LL << 31), "attention_prefill: too many tiles for one launch");
   if (n_tiles == 0) return 0;
   const int group = n_heads / n_kv_heads;
-  dim3 grid(((n_tiles + per_wg - 1) / per_wg) * n_kv_heads), block(256);
+  dim3 grid(n_tiles * n_kv_heads), block(256);
   const bool pow2 = (page_size & (page_size - 1)) == 0;
   const int paging = !pow2 ? 0 : (page_size >= AP_BK ? 2 : 1);
   PYLON_REQUIRE(static_cast<long long>(n_kv_heads) * head_dim * AP_BK < (1LL << 31),
@@ -567,7 +553,7 @@ extern "C" int pylon_attention_prefill(void* out, const void* q, const void* k_c
 #define GO_PAGING(HD, QT, PG)                                                                            \
   hipLaunchKernelGGL((attention_prefill_kernel<HD, QT, PG>), grid, block, 0, stream, (uint16_t*)out,     \
                      (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_table, \
-                     table_width, tiles, n_tiles, per_wg, n_heads, n_kv_heads, group, page_size, window, scale)
+                     table_width, tiles, n_heads, n_kv_heads, group, page_size, window, scale)
 #define GO(HD, QT)                                                                                       \
   do {                                                                                                   \
     if (paging == 2) GO_PAGING(HD, QT, 2);                                                               \
@@ -578,7 +564,7 @@ extern "C" int pylon_attention_prefill(void* out, const void* q, const void* k_c
 #define GO_DIRECT(QT)                                                                                    \
   hipLaunchKernelGGL((attention_prefill_direct_kernel<QT>), grid, block, 0, stream, (uint16_t*)out,      \
                      (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, block_table, \
-                     table_width, tiles, n_tiles, per_wg, n_heads, n_kv_heads, group, page_size, window, scale)
+                     table_width, tiles, n_heads, n_kv_heads, group, page_size, window, scale)
     if (rows == 64) GO_DIRECT(1); else GO_DIRECT(2);
 #undef GO_DIRECT
   } else if (rows == 64) {

@@ -118,18 +118,12 @@ class StepContext:
         more = np.nonzero(self.counts != 1)[0]
         return int(more[0]) if more.size else self.rows
 
-    def count_tiles(self, tokens_per_tile: int, skip_rows: int = 0) -> int:
-        """How many tiles ``token_tiles`` makes."""
-        return int((-(-self.counts[skip_rows:] // tokens_per_tile)).sum())
-
-    def token_tiles(self, tokens_per_tile: int, skip_rows: int = 0, paired: bool = False) -> torch.Tensor:
+    def token_tiles(self, tokens_per_tile: int, skip_rows: int = 0) -> torch.Tensor:
         """int32 ``[n, 4]`` on the device: the step's tokens (without those of the first
         ``skip_rows`` rows) cut into runs of at most ``tokens_per_tile`` consecutive tokens
         of one row, as (index of the first token, count, row, position of the first token),
-        longest context first so that the heaviest tiles start first.  ``paired`` puts the
-        longest beside the shortest, the second longest beside the second shortest and so
-        on, for a kernel whose workgroups take two neighbouring tiles each."""
-        key = (tokens_per_tile, skip_rows, paired)
+        longest context first so that the heaviest tiles start first."""
+        key = (tokens_per_tile, skip_rows)
         tiles = self._tiles.get(key)
         if tiles is None:
             per_row = -(-self.counts // tokens_per_tile)
@@ -143,12 +137,6 @@ class StepContext:
             np.cumsum(self.counts, out=starts[1:])
             table = np.stack([starts[row] + within, count, row, self.starts[row] + within], axis=1)
             order = np.argsort(-(table[:, 3] + table[:, 1]), kind="stable")
-            if paired:
-                n = len(order)
-                mixed = np.empty_like(order)
-                mixed[0::2] = order[: (n + 1) // 2]
-                mixed[1::2] = order[::-1][: n // 2]
-                order = mixed
             host = torch.from_numpy(np.ascontiguousarray(table[order].astype(np.int32)))
             tiles = host.to(self.token_ids.device)
             self._tiles[key] = tiles

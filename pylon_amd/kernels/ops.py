@@ -363,13 +363,6 @@ def prefill_rows(tokens: int, n_heads: int, group: int) -> int:
     return 128 if tokens * n_heads >= 128 * 512 or group > 64 else 64
 
 
-def prefill_tiles_per_workgroup(n_tiles: int, n_kv_heads: int) -> int:
-    """Under a causal mask a tile late in a prompt walks many key blocks and an early one
-    few.  When there are enough tiles that workgroups of two still fill every compute unit,
-    each workgroup takes a long tile and a short one, and all end at about the same time."""
-    return 2 if -(-n_tiles // 2) * n_kv_heads >= 256 else 1
-
-
 PREFILL_MAX_PAGES = 4096  # block-table columns the prefill kernel keeps in LDS
 
 
@@ -384,7 +377,7 @@ def prefill_attention_ok(q: torch.Tensor, k_cache: torch.Tensor, block_table: Op
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_table: torch.Tensor, tiles: torch.Tensor, *, page_size: int,
                       window: Optional[int], scale: float, rows: Optional[int] = None,
-                      out: Optional[torch.Tensor] = None, tiles_per_workgroup: int = 1) -> torch.Tensor:
+                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Paged causal attention of bfloat16 prompt portions on the matrix cores.  ``tiles`` is
     int32 ``[n, 4]``: first token index, token count, block-table row and first position of
     runs of at most ``rows // group`` consecutive tokens of one request; ``rows`` (64 or 128,
@@ -406,7 +399,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _lib.call("pylon_attention_prefill", _dev(out, "out"), _dev(q, "q"), _dev(k_cache, "k_cache"),
               _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
               _dev(tiles, "tiles", torch.int32), tiles.shape[0], n_heads, n_kv_heads, head_dim, page_size,
-              int(window or 0), float(scale), int(rows), int(tiles_per_workgroup), _stream())
+              int(window or 0), float(scale), int(rows), _stream())
     return out
 
 

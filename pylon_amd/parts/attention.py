@@ -107,13 +107,10 @@ class Attention(Part):
                     n_cuts=cuts, out=context[:singles],
                 )
             if singles < ctx.rows:
-                per_tile = rows // group
-                share = ops.prefill_tiles_per_workgroup(ctx.count_tiles(per_tile, singles), spec.n_kv_heads)
-                tiles = ctx.token_tiles(per_tile, skip_rows=singles, paired=share == 2)
+                tiles = ctx.token_tiles(rows // group, skip_rows=singles)
                 ops.attention_prefill(
                     q, cache.k, cache.v, cache.block_table, tiles,
                     page_size=cache.page_size, window=spec.window, scale=spec.scale, rows=rows, out=context,
-                    tiles_per_workgroup=share,
                 )
         else:
             context = ops.paged_attention(

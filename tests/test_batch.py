@@ -31,28 +31,13 @@ def _check_cover(tiles, counts, cached, per_tile, skip):
     assert (seen[starts[skip]:] == 1).all() and (seen[: starts[skip]] == 0).all()
 
 
-def test_tiles_cover_every_token_once_in_both_orders():
+def test_tiles_cover_every_token_once_longest_context_first():
     counts, cached = [1, 1, 37, 5, 64, 130], [9, 0, 0, 31, 16, 3]
     ctx = _step(counts, cached)
     assert ctx.leading_singles == 2
     for per_tile in (4, 16, 32):
         for skip in (0, 2):
-            plain = ctx.token_tiles(per_tile, skip_rows=skip)
-            paired = ctx.token_tiles(per_tile, skip_rows=skip, paired=True)
-            assert len(plain) == len(paired) == ctx.count_tiles(per_tile, skip)
-            _check_cover(plain, counts, cached, per_tile, skip)
-            _check_cover(paired, counts, cached, per_tile, skip)
-            ends = (plain[:, 3] + plain[:, 1]).tolist()
-            assert ends == sorted(ends, reverse=True)  # longest context first
-            # paired: the longest beside the shortest, the second longest beside the second shortest
-            n = len(plain)
-            assert torch.equal(paired[0::2], plain[: (n + 1) // 2])
-            assert torch.equal(paired[1::2], plain.flip(0)[: n // 2])
-
-
-def test_pairing_is_chosen_only_when_the_chip_stays_full():
-    from pylon_amd.kernels import ops
-
-    assert ops.prefill_tiles_per_workgroup(64, 8) == 2   # 2,048 tokens of a 32/8-head model, 128 rows
-    assert ops.prefill_tiles_per_workgroup(32, 8) == 1
-    assert ops.prefill_tiles_per_workgroup(3, 1) == 1
+            tiles = ctx.token_tiles(per_tile, skip_rows=skip)
+            _check_cover(tiles, counts, cached, per_tile, skip)
+            ends = (tiles[:, 3] + tiles[:, 1]).tolist()
+            assert ends == sorted(ends, reverse=True)
