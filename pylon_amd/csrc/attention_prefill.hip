@@ -59,18 +59,14 @@ __device__ __forceinline__ void load_queries(int (&qpos)[QT], bf16x8 (&qf)[QT][H
   }
 }
 
-// One block of 64 keys for one query tile of a wave: s holds the transposed scores (lane
-// (col, grp) has keys kb + 16*kt + 4*grp + r of query column col).  Masks, keeps the
-// running maximum, rescales the NT accumulator tiles when the maximum moves, and returns
-// the probabilities as row operands of the value product: operand slot j of a lane is key
-// 32*kg + 4*grp + j (j < 4) or 32*kg + 16 + 4*grp + (j - 4).  The row sums are not kept
-// here: the caller multiplies the probabilities by a tile of ones as well, so that the last
-// accumulator tile holds, in every column, the sum of exactly the rounded probabilities that
-// weigh the values.
+// One block of 64 keys for one query tile of a wave, first half: s holds the transposed
+// scores (lane (col, grp) has keys kb + 16*kt + 4*grp + r of query column col).  Masks,
+// keeps the running maximum and rescales the NT accumulator tiles when the maximum moves.
+// Returns what to add to scale_log2 * score before the exponential.
 template <int NT>
-__device__ __forceinline__ void softmax_block(floatx4 (&s)[AP_BK / 16], bf16x8 (&pa)[AP_BK / 32], float& m_run,
-                                              floatx4 (&o)[NT], int qp, int kb, bool masked, int window, int grp,
-                                              float scale_log2, float slack) {
+__device__ __forceinline__ float softmax_prepare(floatx4 (&s)[AP_BK / 16], float& m_run, floatx4 (&o)[NT], int qp,
+                                                 int kb, bool masked, int window, int grp, float scale_log2,
+                                                 float slack) {
   if (masked) {
     // key kb + 16*kt + 4*grp + r is seen if it is at most qp and inside the window: compared
     // as 16*kt + r (a constant) against two numbers of this lane
@@ -110,19 +106,24 @@ __device__ __forceinline__ void softmax_block(floatx4 (&s)[AP_BK / 16], bf16x8 (
       for (int nt = 0; nt < NT; ++nt) o[nt][r] *= c;
     }
   }
-  const float shift = (m_run == -INFINITY) ? 0.f : -m_run * scale_log2;
-  float p[AP_BK / 16][4];
+  return (m_run == -INFINITY) ? 0.f : -m_run * scale_log2;
+}
+
+// Second half: the probabilities of keys 32*kg .. 32*kg + 31 as a row operand of the value
+// product.  Operand slot j of a lane is key 32*kg + 4*grp + j (j < 4) or
+// 32*kg + 16 + 4*grp + (j - 4).  The row sums are not kept here: the caller multiplies the
+// probabilities by a tile of ones as well, so that the last accumulator tile holds, in
+// every column, the sum of exactly the rounded probabilities that weigh the values.
+__device__ __forceinline__ bf16x8 probabilities(const floatx4 (&s)[AP_BK / 16], int kg, float scale_log2,
+                                                float shift) {
+  float p[2][4];
 #pragma unroll
-  for (int kt = 0; kt < AP_BK / 16; ++kt)
+  for (int h = 0; h < 2; ++h)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) p[kt][r] = __builtin_amdgcn_exp2f(fmaf(s[kt][r], scale_log2, shift));
-#pragma unroll
-  for (int kg = 0; kg < AP_BK / 32; ++kg) {
-    const u32x4 packed = {pack_bf16(p[2 * kg][0], p[2 * kg][1]), pack_bf16(p[2 * kg][2], p[2 * kg][3]),
-                          pack_bf16(p[2 * kg + 1][0], p[2 * kg + 1][1]),
-                          pack_bf16(p[2 * kg + 1][2], p[2 * kg + 1][3])};
-    pa[kg] = __builtin_bit_cast(bf16x8, packed);
-  }
+    for (int r = 0; r < 4; ++r) p[h][r] = __builtin_amdgcn_exp2f(fmaf(s[2 * kg + h][r], scale_log2, shift));
+  const u32x4 packed = {pack_bf16(p[0][0], p[0][1]), pack_bf16(p[0][2], p[0][3]), pack_bf16(p[1][0], p[1][1]),
+                        pack_bf16(p[1][2], p[1][3])};
+  return __builtin_bit_cast(bf16x8, packed);
 }
 
 // out = acc / sum for a wave's query tiles; a lane holds rows 4*grp + r, element dt*16 + col,
@@ -315,8 +316,12 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
     const bool masked = kb + AP_BK - 1 > pos0 || window > 0;
     bf16x8 pa[QT][AP_BK / 32];
 #pragma unroll
-    for (int qt = 0; qt < QT; ++qt)
-      softmax_block<DT + 1>(s[qt], pa[qt], m_run[qt], o[qt], qpos[qt], kb, masked, window, grp, scale_log2, slack);
+    for (int qt = 0; qt < QT; ++qt) {
+      const float shift = softmax_prepare<DT + 1>(s[qt], m_run[qt], o[qt], qpos[qt], kb, masked, window, grp,
+                                                  scale_log2, slack);
+#pragma unroll
+      for (int kg = 0; kg < AP_BK / 32; ++kg) pa[qt][kg] = probabilities(s[qt], kg, scale_log2, shift);
+    }
 
     // out += P * V, the values in the same order of keys as the probabilities
 #pragma unroll
@@ -487,23 +492,45 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
     __builtin_amdgcn_sched_barrier(0);                                                                 \
     const bool masked = (KB) + AP_BK - 1 > pos0 || window > 0;                                         \
     bf16x8 pa[QT][AP_BK / 32];                                                                         \
-    _Pragma("unroll") for (int qt = 0; qt < QT; ++qt)                                                  \
-      softmax_block<DT + 1>(s[qt], pa[qt], m_run[qt], o[qt], qpos[qt], (KB), masked, window, grp,      \
-                            scale_log2, slack);                                                        \
+    float shift[QT];                                                                                   \
+    _Pragma("unroll") for (int qt = 0; qt < QT; ++qt) {                                                \
+      shift[qt] = softmax_prepare<DT + 1>(s[qt], m_run[qt], o[qt], qpos[qt], (KB), masked, window,     \
+                                          grp, scale_log2, slack);                                     \
+      pa[qt][0] = probabilities(s[qt], 0, scale_log2, shift[qt]);                                      \
+    }                                                                                                  \
     __builtin_amdgcn_sched_barrier(0);                                                                 \
-    _Pragma("unroll") for (int it = 0; it < 2 * DT; ++it) {  /* it = kg * DT + dt */                   \
+    /* the products of the first 32 keys run while the vector unit takes the exponentials of the */    \
+    /* other 32: per output tile two value reads, QT products, and a share of that arithmetic */       \
+    _Pragma("unroll") for (int qt = 0; qt < QT; ++qt)                                                  \
+      pa[qt][1] = probabilities(s[qt], 1, scale_log2, shift[qt]);                                      \
+    _Pragma("unroll") for (int it = 0; it < DT; ++it) {                                                \
+      const bf16x8 vnow = __builtin_bit_cast(                                                          \
+          bf16x8, __builtin_shufflevector(vf[it % AP_VAHEAD][0], vf[it % AP_VAHEAD][1], 0, 1, 2, 3, 4, 5, 6, 7)); \
+      vf[it % AP_VAHEAD][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(                                 \
+          (AP_LDS(s16x4)*)(v_tile + v_at[(it + AP_VAHEAD) % DT] + ((it + AP_VAHEAD) / DT) * 32 * ROW)); \
+      vf[it % AP_VAHEAD][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(                                 \
+          (AP_LDS(s16x4)*)(v_tile + v_at[(it + AP_VAHEAD) % DT] + ((it + AP_VAHEAD) / DT) * 32 * ROW + 16 * ROW)); \
+      _Pragma("unroll") for (int qt = 0; qt < QT; ++qt)                                                \
+        o[qt][it] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[qt][0], vnow, o[qt][it], 0, 0, 0);      \
+    }                                                                                                  \
+    _Pragma("unroll") for (int it = 0; it < DT; ++it) {                                                \
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  /* LDS reads */                              \
+      __builtin_amdgcn_sched_group_barrier(0x008, QT, 0); /* matrix products */                        \
+      __builtin_amdgcn_sched_group_barrier(0x402, (20 * QT + DT - 1) / DT, 0); /* vector arithmetic */ \
+    }                                                                                                  \
+    __builtin_amdgcn_sched_barrier(0);                                                                 \
+    _Pragma("unroll") for (int it = DT; it < 2 * DT; ++it) {                                           \
       const bf16x8 vnow = __builtin_bit_cast(                                                          \
           bf16x8, __builtin_shufflevector(vf[it % AP_VAHEAD][0], vf[it % AP_VAHEAD][1], 0, 1, 2, 3, 4, 5, 6, 7)); \
       if (it + AP_VAHEAD < 2 * DT) {                                                                   \
-        const int nkg = (it + AP_VAHEAD) / DT, ndt = (it + AP_VAHEAD) % DT;                            \
         vf[it % AP_VAHEAD][0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(                               \
-            (AP_LDS(s16x4)*)(v_tile + v_at[ndt] + nkg * 32 * ROW));                                    \
+            (AP_LDS(s16x4)*)(v_tile + v_at[(it + AP_VAHEAD) % DT] + 32 * ROW));                        \
         vf[it % AP_VAHEAD][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(                               \
-            (AP_LDS(s16x4)*)(v_tile + v_at[ndt] + nkg * 32 * ROW + 16 * ROW));                         \
+            (AP_LDS(s16x4)*)(v_tile + v_at[(it + AP_VAHEAD) % DT] + 32 * ROW + 16 * ROW));             \
       }                                                                                                \
       __builtin_amdgcn_sched_barrier(0);                                                               \
       _Pragma("unroll") for (int qt = 0; qt < QT; ++qt)                                                \
-        o[qt][it % DT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[qt][it / DT], vnow, o[qt][it % DT], 0, 0, 0); \
+        o[qt][it % DT] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa[qt][1], vnow, o[qt][it % DT], 0, 0, 0); \
       __builtin_amdgcn_sched_barrier(0);                                                               \
     }                                                                                                  \
     _Pragma("unroll") for (int kg = 0; kg < AP_BK / 32; ++kg)                                          \
