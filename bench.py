@@ -193,6 +193,38 @@ def prefill_run(runner, cfg, repeats: int, seed: int):
     return times[len(times) // 2]
 
 
+def mixed_run(runner, cfg, batch: int, prompt_len: int, repeats: int, seed: int) -> float:
+    """Seconds of one mixed step: one token for each of ``batch`` requests that hold
+    ``prompt_len`` tokens, beside a PREFILL_TOKENS portion of a new prompt, with greedy
+    sampling of the batch + 1 wanted rows on the device; the median."""
+    import numpy as np
+    import torch
+
+    from pylon_amd.engine import StepEntry
+    from pylon_amd.sampling import Sampler, Sampling
+
+    rng = np.random.default_rng(seed)
+    sampler = Sampler(runner.model.device)
+    greedy = [(Sampling(temperature=0.0), 0)] * (batch + 1)
+    seqs = [runner.open(f"m{batch}-{i}") for i in range(batch)]
+    feed_prompts(runner, sampler, seqs, [rng.integers(0, cfg.vocab_size, prompt_len).tolist() for _ in seqs])
+    times = []
+    for r in range(repeats + 1):
+        fresh = runner.open(f"mixed-prompt-{r}")
+        entries = [StepEntry(s, [int(rng.integers(0, cfg.vocab_size))], [0]) for s in seqs]
+        entries.append(StepEntry(fresh, rng.integers(0, cfg.vocab_size, PREFILL_TOKENS).tolist(), [PREFILL_TOKENS - 1]))
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        out = runner.step(entries)
+        sampler.launch(out, greedy, chosen=runner.chosen, place=runner.logit_slots).result()
+        times.append(time.perf_counter() - started)
+        runner.close(fresh)
+    for s in seqs:
+        runner.close(s)
+    times = sorted(times[1:])
+    return times[len(times) // 2]
+
+
 def engine_run(runner, cfg, batch: int, seed: int, prompt_len: int = PROMPT_LEN) -> float:
     """The same work through the scheduler: ``batch`` requests of ``prompt_len`` random ids and
     NEW_TOKENS greedy tokens each, queued at once; generated tokens per second from the first
@@ -231,6 +263,8 @@ def main() -> int:
     parser.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     parser.add_argument("--no-prefill", action="store_true")
+    parser.add_argument("--mixed", action="store_true",
+                        help="also time a step of --batch decoded tokens beside a 2,048-token prompt portion")
     parser.add_argument("--prefill-only", action="store_true",
                         help="only the prefill measurement (for profiling); prints its part of the record")
     args = parser.parse_args()
@@ -257,8 +291,8 @@ def main() -> int:
     if max_batch * pages_per_request * page_bytes > 100e9:
         longest = max(prompt_len + steps + args.warmup + 1, PREFILL_TOKENS)
         pages_per_request = -(-longest // PAGE_SIZE) + 1
-    runner, cfg = build_runner(shape, layers, args.dtype, max_requests=max_batch,
-                               num_pages=max_batch * pages_per_request, graphs=not args.no_graphs)
+    runner, cfg = build_runner(shape, layers, args.dtype, max_requests=max_batch + 1,
+                               num_pages=(max_batch + 1) * pages_per_request, graphs=not args.no_graphs)
     dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
     if args.prefill_only:
         seconds = prefill_run(runner, cfg, repeats=5, seed=2)
@@ -301,6 +335,9 @@ def main() -> int:
         record["prefill"] = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
                              "ms": round(1e3 * seconds, 3),
                              "frac": round(flops / seconds / PEAK_FLOPS[dtype_key], 4)}
+    if args.mixed:
+        seconds = mixed_run(runner, cfg, args.batch, prompt_len, repeats=5, seed=4)
+        record["mixed"] = {"decodes": args.batch, "chunk": PREFILL_TOKENS, "ms": round(1e3 * seconds, 3)}
     if not args.no_points:
         points = {}
         for batch in (1, 64):
