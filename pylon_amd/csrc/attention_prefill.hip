@@ -4,16 +4,21 @@
 // A workgroup of four wavefronts takes one tile of consecutive tokens of one request and
 // one key/value head, together with all query heads of that head's group: a (token, head)
 // pair is one of up to 64 or 128 query rows, 16 or 32 per wave.  Keys and values are walked
-// 64 at a time.  While one block of keys is being used, the next is already on its way
-// from the cache into registers; at the top of an iteration the registers go to LDS: the
-// 64 keys row-major, the 64 values transposed (a thread holds eight elements of four
+// 64 at a time.  Scores are computed transposed (keys as rows, queries as columns): the
+// result registers of a score tile then already have the layout the row operand of the
+// value product needs, and the running maximum of a query lives in the lanes of its
+// column.  Scores, softmax and the output accumulators are float; exponentials are exp2
+// with scale*log2(e) folded into one multiply-add; the sums of the probabilities come out
+// of the matrix cores (a product with a tile of ones).
+//
+// Two kernels share this arithmetic and differ in how a block of keys and values reaches
+// the matrix cores.  The general one (attention_prefill_kernel) fetches the next block into
+// registers while the current one is used and writes it to LDS at the top of an iteration:
+// the 64 keys row-major, the 64 values transposed (a thread holds eight elements of four
 // consecutive keys and writes, per element, the four keys as one 8-byte word), so that a
-// lane reads the column operand of the value product as two 8-byte words.  Scores are
-// computed transposed (keys as rows, queries as columns): the result registers of a score
-// tile then already have the layout the row operand of the value product needs, and the
-// running maximum and sum of a query live in the lanes of its column.  Scores, softmax and
-// the output accumulators are float; exponentials are exp2 with scale*log2(e) folded into
-// one multiply-add.
+// lane reads the column operand of the value product as two 8-byte words.  The one for head
+// size 128 and block-aligned pages (attention_prefill_direct_kernel, further down) lets the
+// memory system write LDS itself and transposes on the way out of LDS.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
