@@ -377,7 +377,8 @@ def test_attention_decode_for_a_large_batch(ops):
 
 @pytest.mark.parametrize("geom", [(8, 2, 128, 64, None), (4, 4, 64, 16, None), (12, 2, 128, 32, 100),
                                   (5, 1, 256, 16, None), (3, 3, 64, 256, 37), (16, 1, 128, 64, None),
-                                  (8, 4, 128, 48, None), (6, 2, 64, 80, 90)])
+                                  (8, 4, 128, 48, None), (6, 2, 64, 80, 90), (8, 2, 128, 64, 90),
+                                  (6, 3, 128, 128, 200), (5, 5, 128, 256, None)])
 @pytest.mark.parametrize("rows", [64, 128])
 def test_attention_prefill(ops, geom, rows):
     """Portions of several requests at once: starting inside a page, a one-token portion, a
