@@ -438,14 +438,16 @@ def test_attention_prefill(ops, geom, rows):
     assert float((got.float() - ref.float()).abs().max()) <= 3e-2
 
 
-@pytest.mark.parametrize("kernel", ["general_f32", "general_bf16", "decode", "prefill"])
+@pytest.mark.parametrize("kernel", ["general_f32", "general_bf16", "decode", "prefill", "prefill_direct"])
 def test_attention_finds_one_far_key_among_hundreds(ops, kernel):
     # Random keys would hide a key that is skipped; here one far key matches the query
     # exactly and strongly, so the output must be (almost) that key's value.
     dtype = torch.float32 if kernel == "general_f32" else torch.bfloat16
     nh, nkv, hd, page = 2, 1, 64, 16
+    if kernel == "prefill_direct":  # the prompt kernel that loads whole blocks of a page into LDS
+        hd, page = 128, 64
     n = 777
-    for far in (0, 15, 16, 400, 776 - 64, 775, 776):
+    for far in (0, 15, 16, 63, 64, 400, 776 - 64, 767, 768, 775, 776):
         kc = (rnd((50, page, nkv, hd), 17) * 0.01).to(dtype)
         vc = rnd((50, page, nkv, hd), 18).to(dtype)
         table = torch.arange(49, -1, -1, dtype=torch.int32).reshape(1, 50)
@@ -457,7 +459,7 @@ def test_attention_finds_one_far_key_among_hundreds(ops, kernel):
         args = (q.to(DEV), kc.to(DEV), vc.to(DEV), table.to(DEV))
         if kernel == "decode":
             got = ops.attention_decode(*args, row, pos, page_size=page, window=None, scale=1.0, n_splits=8)
-        elif kernel == "prefill":
+        elif kernel.startswith("prefill"):
             tiles = torch.tensor([[0, 1, 0, n - 1]], dtype=torch.int32, device=DEV)
             got = ops.attention_prefill(*args, tiles, page_size=page, window=None, scale=1.0)
         else:
@@ -465,10 +467,12 @@ def test_attention_finds_one_far_key_among_hundreds(ops, kernel):
         assert torch.allclose(got[0, 0].float().cpu(), vc[page_id, off, 0].float(), atol=2e-2), (kernel, far)
 
 
-@pytest.mark.parametrize("kernel", ["general", "decode", "prefill"])
+@pytest.mark.parametrize("kernel", ["general", "decode", "prefill", "prefill_direct"])
 def test_attention_window_edge_fast_kernels(ops, kernel):
     # the key at distance `window` must be invisible, the one at distance window-1 visible
     nh, nkv, hd, page, window = 1, 1, 64, 16, 37
+    if kernel == "prefill_direct":
+        hd, page = 128, 64
     dtype = torch.bfloat16
     kc = torch.zeros((8, page, nkv, hd), dtype=dtype)
     vc = rnd((8, page, nkv, hd), 20, dtype)
@@ -483,7 +487,7 @@ def test_attention_window_edge_fast_kernels(ops, kernel):
         args = (q.to(DEV), k2.to(DEV), vc.to(DEV), table.to(DEV))
         if kernel == "decode":
             got = ops.attention_decode(*args, row, p, page_size=page, window=window, scale=1.0, n_splits=2)
-        elif kernel == "prefill":
+        elif kernel.startswith("prefill"):
             tiles = torch.tensor([[0, 1, 0, pos]], dtype=torch.int32, device=DEV)
             got = ops.attention_prefill(*args, tiles, page_size=page, window=window, scale=1.0)
         else:
