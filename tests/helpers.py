@@ -49,10 +49,17 @@ TINY_D = _qwen3(
     intermediate_size=208, vocab_size=331, rope_theta=250000.0, rms_norm_eps=2e-6,
     tie_word_embeddings=True, max_position_embeddings=4096,
 )
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+# E has the head size of every published Qwen3 model, 128: with pages of 64 tokens its prompt
+# portions run on the attention kernel that loads whole blocks of a page straight into LDS.
+TINY_E = _qwen3(
+    num_hidden_layers=2, hidden_size=72, num_attention_heads=3, num_key_value_heads=1, head_dim=128,
+    intermediate_size=144, vocab_size=277, rope_theta=1000000.0, rms_norm_eps=1e-5,
+    tie_word_embeddings=False, max_position_embeddings=1024,
+)
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
 # A has unit norm weights; the others draw them, so that a kernel ignoring a norm weight fails.
-NORM_JITTER = {"A": 0.0, "B": 0.2, "C": 0.2, "D": 0.2}
-SEEDS = {"A": 11, "B": 23, "C": 37, "D": 41}
+NORM_JITTER = {"A": 0.0, "B": 0.2, "C": 0.2, "D": 0.2, "E": 0.2}
+SEEDS = {"A": 11, "B": 23, "C": 37, "D": 41, "E": 53}
 
 
 def make_model_folder(tmp: Path, name: str, *, dtype: str = "float32", config=None, seed=None,

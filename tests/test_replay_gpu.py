@@ -30,7 +30,7 @@ BOUND = {"float32": 2e-5, "bfloat16": 2e-2}
 CUT_BOUND = {"float32": 0.0, "bfloat16": 1e-2}
 
 LENGTHS = {"A": (5, 17, 33, 97, 128), "B": (1, 31, 64, 100, 200, 256), "C": (40, 333, 70, 129),
-           "D": (2, 150, 2100, 65)}
+           "D": (2, 150, 2100, 65), "E": (3, 200, 70, 450)}
 
 
 def requests_for(name):
@@ -105,7 +105,7 @@ CUTTINGS = {
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_every_cutting_matches_the_plain_implementation(folders, name, dtype):
     folder, cfg, want = folders[name, dtype]
     reqs = requests_for(name)
