@@ -18,6 +18,7 @@ class PylonConfig:
     model_path: Optional[str] = None
     dtype: str = "bfloat16"
     max_gpu_utilization: float = 0.90
+    weight_headroom_ratio: float = 0.20
     kv_cache_headroom_ratio: float = 0.20
     prefill_chunk_size: int = 2048
     max_batch_size: int = 32
@@ -37,8 +38,9 @@ class PylonConfig:
             raise ValueError("dtype must be bfloat16 or float32.")
         if not math.isfinite(self.max_gpu_utilization) or not 0 < self.max_gpu_utilization <= 1:
             raise ValueError("max_gpu_utilization must be greater than 0 and at most 1.")
-        if not 0 <= self.kv_cache_headroom_ratio < 1:
-            raise ValueError("kv_cache_headroom_ratio must be at least 0 and less than 1.")
+        for name in ("weight_headroom_ratio", "kv_cache_headroom_ratio"):
+            if not 0 <= getattr(self, name) < 1:
+                raise ValueError(f"{name} must be at least 0 and less than 1.")
         for name in ("prefill_chunk_size", "page_size"):
             value = getattr(self, name)
             if not isinstance(value, int) or isinstance(value, bool) or value < 1:
@@ -73,6 +75,7 @@ def get_config(**overrides) -> PylonConfig:
         model_path=os.getenv("PYLON_MODEL_PATH") or None,
         dtype=os.getenv("PYLON_DTYPE", "bfloat16"),
         max_gpu_utilization=float(os.getenv("PYLON_MAX_GPU_UTILIZATION", "0.90")),
+        weight_headroom_ratio=float(os.getenv("PYLON_WEIGHT_HEADROOM_RATIO", "0.20")),
         kv_cache_headroom_ratio=float(os.getenv("PYLON_KV_CACHE_HEADROOM_RATIO", "0.20")),
         prefill_chunk_size=int(os.getenv("PYLON_PREFILL_CHUNK_SIZE", "2048")),
         max_batch_size=int(os.getenv("PYLON_MAX_BATCH_SIZE", "32")),

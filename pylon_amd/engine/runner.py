@@ -8,6 +8,7 @@ be replayed from a HIP graph.
 """
 from __future__ import annotations
 
+import math
 from pathlib import Path
 from typing import Hashable, Optional, Sequence as Seq
 
@@ -29,6 +30,24 @@ def resolve_dtype(dtype) -> torch.dtype:
         return _DTYPES[dtype]
     except KeyError:
         raise ValueError("dtype must be bfloat16 or float32") from None
+
+
+def weight_bytes(spec, dtype: torch.dtype) -> int:
+    """Bytes of every parameter of a model of this spec, counted without allocating it."""
+    model = Model(spec, dtype=dtype, device="meta")
+    return sum(owner.params[name].numel() * owner.params[name].element_size()
+               for _, owner, name in model.named_params())
+
+
+def check_weights_fit(needed: int, free: int, total: int, config, what) -> None:
+    """Refuse a model whose weights, with their headroom, do not fit under the utilisation
+    limit (/root/reference/src/pylon/kv/budget.py:49-68, model/loader.py:59-72)."""
+    required = int(needed * (1 + config.weight_headroom_ratio))
+    available = max(0, math.floor(total * config.max_gpu_utilization) - (total - free))
+    if required > available:
+        raise RuntimeError(
+            f"Refusing to load {what}: weights and headroom need {required:,} bytes; "
+            f"{available:,} bytes are available under the GPU utilization limit.")
 
 
 class Runner:
@@ -71,7 +90,10 @@ class Runner:
         if not torch.cuda.is_available():
             raise RuntimeError("A GPU is required: the step function has no CPU path.")
         arch, model_config = load_model_config(config.model_path)
-        model = Model(arch.model_spec(model_config), dtype=resolve_dtype(config.dtype), device=device)
+        spec = arch.model_spec(model_config)
+        free, total = torch.cuda.mem_get_info(torch.device(device))
+        check_weights_fit(weight_bytes(spec, resolve_dtype(config.dtype)), free, total, config, config.model_path)
+        model = Model(spec, dtype=resolve_dtype(config.dtype), device=device)
         load_weights(model, arch, model_config, Path(config.model_path))
         num_pages = config.num_pages
         if num_pages is None:

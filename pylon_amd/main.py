@@ -26,6 +26,7 @@ def _add_serving_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--max-queue-size", type=int)
     p.add_argument("--batch-wait-ms", type=float)
     p.add_argument("--max-gpu-utilization", type=float)
+    p.add_argument("--weight-headroom-ratio", type=float)
     p.add_argument("--kv-cache-headroom-ratio", type=float)
     p.add_argument("--admit-skip", type=int)
     p.add_argument("--page-size", type=int)
@@ -54,6 +55,7 @@ def _generate(args) -> int:
         model_path=args.model, dtype=args.dtype, prefill_chunk_size=args.prefill_chunk_size,
         max_batch_size=args.max_batch_size, max_queue_size=args.max_queue_size,
         batch_wait_ms=args.batch_wait_ms, max_gpu_utilization=args.max_gpu_utilization,
+        weight_headroom_ratio=args.weight_headroom_ratio,
         kv_cache_headroom_ratio=args.kv_cache_headroom_ratio, admit_skip=args.admit_skip,
         page_size=args.page_size, num_pages=args.num_pages, cuda_graphs=args.cuda_graphs,
         run_ahead=args.run_ahead,

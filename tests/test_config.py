@@ -120,11 +120,12 @@ def test_serving_config_defaults_and_checks(monkeypatch):
     cfg = PylonConfig()
     # the reference's defaults (/root/reference/src/pylon/config.py:14-26)
     assert (cfg.prefill_chunk_size, cfg.max_batch_size, cfg.max_queue_size, cfg.batch_wait_ms,
-            cfg.max_gpu_utilization, cfg.kv_cache_headroom_ratio, cfg.cuda_graphs, cfg.admit_skip) == (
-        2048, 32, 32, 2.0, 0.90, 0.20, False, 4)
+            cfg.max_gpu_utilization, cfg.weight_headroom_ratio, cfg.kv_cache_headroom_ratio, cfg.cuda_graphs,
+            cfg.admit_skip) == (2048, 32, 32, 2.0, 0.90, 0.20, 0.20, False, 4)
     for bad in (dict(prefill_chunk_size=0), dict(max_batch_size=0), dict(max_queue_size=0),
                 dict(batch_wait_ms=-1), dict(max_gpu_utilization=0), dict(max_gpu_utilization=1.5),
-                dict(kv_cache_headroom_ratio=1.0), dict(admit_skip=-1), dict(admit_skip=True),
+                dict(kv_cache_headroom_ratio=1.0), dict(weight_headroom_ratio=-0.1), dict(admit_skip=-1),
+                dict(admit_skip=True),
                 dict(dtype="float16"), dict(page_size=24)):
         with pytest.raises(ValueError):
             PylonConfig(**bad)
@@ -137,3 +138,26 @@ def test_serving_config_defaults_and_checks(monkeypatch):
     monkeypatch.setenv("PYLON_CUDA_GRAPHS", "yes")
     with pytest.raises(ValueError, match="must be true, false, 1, or 0"):
         get_config()
+
+
+def test_weights_must_fit_under_the_utilisation_limit():
+    # /root/reference/src/pylon/kv/budget.py:49-68: weights times (1 + headroom) against
+    # utilisation * total minus what is occupied
+    import torch
+
+    from pylon_amd.engine.runner import check_weights_fit, weight_bytes
+
+    raw = dict(TINY_A)
+    arch = resolve(raw)
+    spec = arch.model_spec(arch.parse_config(raw))
+    # embedding 256*64 (tied head), two layers of (64 + 64 + 16 + 16) norm weights,
+    # qkv (64 + 2*32)*64, out 64*64, gate/up 2*128*64, down 64*128, and the final norm
+    per_layer = 64 + 64 + 16 + 16 + 128 * 64 + 64 * 64 + 256 * 64 + 64 * 128
+    norms = 2 * (64 + 64 + 16 + 16) + 64
+    assert weight_bytes(spec, torch.bfloat16) == 2 * (256 * 64 + 2 * per_layer + 64 - norms) + 4 * norms
+    total = 1000
+    check_weights_fit(600, free=total, total=total, config=PylonConfig(), what="m")  # 720 <= 900
+    with pytest.raises(RuntimeError, match="weights and headroom need 960 bytes; 900 bytes are available"):
+        check_weights_fit(800, free=total, total=total, config=PylonConfig(), what="m")
+    with pytest.raises(RuntimeError, match="720 bytes; 700 bytes"):
+        check_weights_fit(600, free=800, total=total, config=PylonConfig(), what="m")  # 200 occupied
