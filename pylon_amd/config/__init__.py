@@ -5,6 +5,7 @@ from .registry import (
     architecture_name,
     load_model_config,
     read_config_json,
+    read_stop_token_ids,
     register_architecture,
     registered_architectures,
     resolve,
@@ -28,6 +29,7 @@ __all__ = [
     "architecture_name",
     "load_model_config",
     "read_config_json",
+    "read_stop_token_ids",
     "register_architecture",
     "registered_architectures",
     "resolve",

@@ -93,3 +93,19 @@ def load_model_config(folder):
     raw = read_config_json(folder)
     arch = resolve(raw)
     return arch, arch.parse_config(raw)
+
+
+def read_stop_token_ids(folder) -> tuple:
+    """The ids that end a generation: ``eos_token_id`` (a number or a list) of the folder's
+    ``generation_config.json`` if there is one, else of its ``config.json``; none if neither
+    names any (/root/reference/src/pylon/model/tokenizer.py:24-38, which insists on one)."""
+    folder = Path(folder)
+    for name in ("generation_config.json", "config.json"):
+        path = folder / name
+        if not path.is_file():
+            continue
+        eos = json.loads(path.read_text()).get("eos_token_id")
+        if eos is None:
+            continue
+        return (int(eos),) if isinstance(eos, int) else tuple(int(token_id) for token_id in eos)
+    return ()

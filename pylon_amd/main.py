@@ -79,7 +79,14 @@ def _generate(args) -> int:
     else:
         engine = Engine(config)
     try:
-        eos = _parse_ids(args.eos_token_id) if args.eos_token_id else getattr(engine.runner.config, "eos_token_id", None)
+        if args.eos_token_id:
+            eos = _parse_ids(args.eos_token_id)
+        elif args.model:
+            from .config import read_stop_token_ids
+
+            eos = read_stop_token_ids(args.model) or None
+        else:
+            eos = getattr(engine.runner.config, "eos_token_id", None)
         results = engine.generate(prompts, sampling, eos)
     finally:
         engine.close()

@@ -161,3 +161,17 @@ def test_weights_must_fit_under_the_utilisation_limit():
         check_weights_fit(800, free=total, total=total, config=PylonConfig(), what="m")
     with pytest.raises(RuntimeError, match="720 bytes; 700 bytes"):
         check_weights_fit(600, free=800, total=total, config=PylonConfig(), what="m")  # 200 occupied
+
+
+def test_stop_ids_come_from_generation_config_before_config(tmp_path):
+    # /root/reference/src/pylon/model/tokenizer.py:24-38
+    from pylon_amd.config import read_stop_token_ids
+
+    (tmp_path / "config.json").write_text(json.dumps(dict(TINY_A, eos_token_id=7)))
+    assert read_stop_token_ids(tmp_path) == (7,)
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": [3, 9]}))
+    assert read_stop_token_ids(tmp_path) == (3, 9)
+    (tmp_path / "generation_config.json").write_text(json.dumps({"temperature": 0.6}))
+    assert read_stop_token_ids(tmp_path) == (7,)
+    (tmp_path / "config.json").write_text(json.dumps(TINY_A))
+    assert read_stop_token_ids(tmp_path) == ()
