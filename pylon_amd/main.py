@@ -9,6 +9,7 @@ still work as defaults), and the commands run on token ids:
     python main.py random-model --config config.json --seed 0 --out DIR
     python main.py replay --model DIR --dtype float32 --out DIR --max-tokens N  < steps.jsonl
     python main.py bench [bench.py's options]
+    python main.py selftest
 """
 from __future__ import annotations
 
@@ -142,8 +143,24 @@ def main(argv=None) -> None:
                          add_help=False)
     ben.add_argument("rest", nargs=argparse.REMAINDER)
 
+    sub.add_parser("selftest", help="generate a few tokens with a tiny random model and compare them with "
+                                    "the plain implementation (needs the repository's tests folder)")
+
     args = parser.parse_args(argv)
-    if args.command == "generate":
+    if args.command == "selftest":
+        root = Path(__file__).resolve().parent.parent
+        if str(root) not in sys.path:
+            sys.path.insert(0, str(root))
+        import torch
+
+        if not torch.cuda.is_available():
+            print("A GPU is required.", file=sys.stderr)
+            sys.exit(1)
+        import __graft_entry__
+
+        __graft_entry__.smoke()
+        code = 0
+    elif args.command == "generate":
         code = _generate(args)
     elif args.command == "random-model":
         code = _random_model(args)
