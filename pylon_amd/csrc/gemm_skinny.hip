@@ -3,7 +3,9 @@
 //
 // A workgroup of 4 or 8 wavefronts owns 16 rows of w (16 output columns), or 32 rows as two
 // tiles for matrices with many rows (the rows of x it loads then serve both; measured
-// 151 us against 165 us for a 151936 x 2560 matrix).  The waves take
+// 151 us against 165 us for a 151936 x 2560 matrix), or, on request, 64 rows as four tiles
+// (for 17 to 64 rows of x, which are two to four tiles themselves and would else be most of
+// what a workgroup reads).  The waves take
 // turns along K in steps of 64: in a step a wave reads one full 128-byte line of each of
 // its 16 rows, as two loads that each cover a contiguous 64-byte half of every line.
 // All loads of a batch of steps are issued before the first product, so a wave with few
@@ -40,17 +42,19 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
-// RT: 16-row tiles of w per workgroup (with GLU: one tile of gate rows and one of up rows)
+// RT: 16-row tiles of w per workgroup (with GLU: RT tiles of gate rows and RT of up rows).
+// A wave multiplies every tile of w with every tile of x, so RT tiles of w pay for the rows of
+// x once: with many rows of x, x (read from the cache) would else be most of the traffic.
 template <int MT, int WAVES, bool GLU, int RT, typename TO>
 __global__ __launch_bounds__(WAVES* PYLON_WAVE) void gemm_skinny_kernel(
     TO* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int M, int N,
     int K, long long ldx, long long ldw, long long ldo, long long part_stride) {
-  constexpr int TILES = GLU ? 2 : RT;  // row tiles of w per workgroup
+  constexpr int TILES = GLU ? 2 * RT : RT;  // row tiles of w per workgroup
   __shared__ floatx4 red[WAVES][TILES][MT][PYLON_WAVE];
   const int lane = threadIdx.x & (PYLON_WAVE - 1);
   const int wave = threadIdx.x / PYLON_WAVE;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16 * (GLU ? 1 : RT);
+  const int n0 = blockIdx.x * 16 * RT;
   const int parts = gridDim.y, part = blockIdx.y;
 
   const int steps = (K + SK_STEP - 1) / SK_STEP;
@@ -61,9 +65,9 @@ __global__ __launch_bounds__(WAVES* PYLON_WAVE) void gemm_skinny_kernel(
   const uint16_t* wp[TILES];
 #pragma unroll
   for (int j = 0; j < TILES; ++j) {
-    const int row = GLU ? n0 + r : n0 + 16 * j + r;
+    const int row = n0 + 16 * (j % RT) + r;
     const int wrow = (row < N) ? row : N - 1;
-    wp[j] = w + static_cast<size_t>((GLU && j == 1) ? N + wrow : wrow) * ldw;
+    wp[j] = w + static_cast<size_t>((GLU && j >= RT) ? N + wrow : wrow) * ldw;
   }
   const uint16_t* xp[MT];
 #pragma unroll
@@ -78,7 +82,8 @@ __global__ __launch_bounds__(WAVES* PYLON_WAVE) void gemm_skinny_kernel(
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[j][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  constexpr int BATCH = (MT == 1) ? (TILES == 2 ? 5 : 10) : (MT == 2 ? 4 : 2) / (TILES == 2 && !GLU ? 2 : 1);
+  // steps whose loads are issued together: about 16 loads of 16 bytes per lane and half step
+  constexpr int BATCH = (MT == 1) ? (TILES == 2 ? 5 : 10) : (16 / (TILES + MT) > 0 ? 16 / (TILES + MT) : 1);
   for (int s0 = s_begin + wave; s0 < s_end; s0 += WAVES * BATCH) {
     bf16x8 a[BATCH][TILES][2], b[BATCH][MT][2];
 #pragma unroll
@@ -128,10 +133,12 @@ __global__ __launch_bounds__(WAVES* PYLON_WAVE) void gemm_skinny_kernel(
       TO* dst = out + static_cast<size_t>(part) * part_stride + static_cast<size_t>(m) * ldo;
       if (GLU) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int n = n0 + 4 * g + i;
-          if (n < N) dst[n] = from_float<TO>(silu_f(sum[0][i]) * sum[TILES - 1][i]);
-        }
+        for (int j = 0; j < RT; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int n = n0 + 16 * j + 4 * g + i;
+            if (n < N) dst[n] = from_float<TO>(silu_f(sum[j][i]) * sum[RT + j][i]);
+          }
       } else {
 #pragma unroll
         for (int j = 0; j < TILES; ++j)
@@ -149,7 +156,7 @@ template <int MT, int WAVES, bool GLU, int RT>
 static void launch_skinny(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                           long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
                           hipStream_t stream) {
-  constexpr int ROWS = 16 * (GLU ? 1 : RT);
+  constexpr int ROWS = 16 * RT;
   dim3 grid((N + ROWS - 1) / ROWS, parts), block(WAVES * PYLON_WAVE);
   if (out_dtype == PYLON_F32)
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, WAVES, GLU, RT, float>), grid, block, 0, stream, (float*)out,
@@ -162,12 +169,19 @@ static void launch_skinny(void* out, int out_dtype, const void* x, const void* w
 template <int MT>
 static void launch_skinny_mt(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                              long long ldx, long long ldw, long long ldo, int parts,
-                             long long part_stride, int glu, hipStream_t stream) {
+                             long long part_stride, int glu, int row_tiles, hipStream_t stream) {
   // Four waves measured faster than eight at every shape of a 4B-class decoder; the
   // eight-wave form is kept for very long K only.
   const int steps = (K + SK_STEP - 1) / SK_STEP / parts;
   const bool wide = steps >= 512;
 #define GO(W, G, R) launch_skinny<MT, W, G, R>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream)
+  if constexpr (MT > 1) {
+    // Several tiles of x: four tiles of w share them if the caller asks for it.
+    if (row_tiles == 4 && !glu) {
+      GO(4, false, 4);
+      return;
+    }
+  }
   if (glu) {
     if (wide) GO(8, true, 1); else GO(4, true, 1);
   } else if (MT == 1 && parts == 1 && N >= 4096) {
@@ -185,8 +199,10 @@ static void launch_skinny_mt(void* out, int out_dtype, const void* x, const void
 // and no glu).
 extern "C" int pylon_gemm_skinny(void* out, int out_dtype, const void* x, const void* w, int M, int N,
                                  int K, long long ldx, long long ldw, long long ldo, int parts,
-                                 long long part_stride, int glu, hipStream_t stream) {
+                                 long long part_stride, int glu, int row_tiles, hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(out_dtype), "gemm_skinny: unknown output dtype");
+  PYLON_REQUIRE(row_tiles == 0 || (row_tiles == 4 && !glu),
+                "gemm_skinny: row_tiles is 0 (automatic) or, without glu, 4; got %d", row_tiles);
   PYLON_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: takes at most 64 rows, got %d", M);
   PYLON_REQUIRE(N > 0 && K > 0, "gemm_skinny: bad sizes N=%d K=%d", N, K);
   PYLON_REQUIRE(K % 8 == 0, "gemm_skinny: K=%d must be a multiple of 8", K);
@@ -201,10 +217,10 @@ extern "C" int pylon_gemm_skinny(void* out, int out_dtype, const void* x, const 
                 "gemm_skinny: partial results overlap");
   if (M == 0) return 0;
   switch ((M + 15) / 16) {
-    case 1: launch_skinny_mt<1>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, stream); break;
-    case 2: launch_skinny_mt<2>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, stream); break;
-    case 3: launch_skinny_mt<3>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, stream); break;
-    default: launch_skinny_mt<4>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, stream); break;
+    case 1: launch_skinny_mt<1>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, row_tiles, stream); break;
+    case 2: launch_skinny_mt<2>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, row_tiles, stream); break;
+    case 3: launch_skinny_mt<3>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, row_tiles, stream); break;
+    default: launch_skinny_mt<4>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, row_tiles, stream); break;
   }
   PYLON_LAUNCHED("gemm_skinny");
 }

@@ -448,12 +448,14 @@ def skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
 
 
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype = torch.bfloat16,
-                parts: int = 1, glu: bool = False) -> torch.Tensor:
+                parts: int = 1, glu: bool = False, row_tiles: int = 0) -> torch.Tensor:
     """``x @ weight.T`` for at most 64 rows of bfloat16 ``x``, streaming ``weight`` once.
 
     ``parts > 1`` cuts K into that many ranges and returns float32 partial results
     ``[parts, M, N]`` for the consumer to add.  ``glu``: ``weight`` is a fused
     ``[2N, K]`` gate/up matrix and the result is ``silu(x @ gate.T) * (x @ up.T)``.
+    ``row_tiles=4`` (more than 16 rows, no ``glu``): a workgroup takes 64 rows of ``weight``
+    instead of 16, so that the rows of ``x`` it reads serve four times as many.
     """
     if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
         raise KernelError(f"gemm_skinny: cannot multiply {tuple(x.shape)} by the transpose of {tuple(weight.shape)}")
@@ -472,7 +474,7 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype
     else:
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     _lib.call("pylon_gemm_skinny", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), weight.data_ptr(),
-              m, n, k, x.stride(0), weight.stride(0), n, parts, m * n, 1 if glu else 0, _stream())
+              m, n, k, x.stride(0), weight.stride(0), n, parts, m * n, 1 if glu else 0, int(row_tiles), _stream())
     return out
 
 
@@ -512,7 +514,19 @@ def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: tor
     residual norm adds."""
     if skinny_ok(x, weight):
         return gemm_skinny(x, weight, out_dtype=out_dtype, parts=k_parts(*weight.shape))
+    if _streaming_ok(x, weight, 64) and deep_or_small(*weight.shape):
+        n, k = weight.shape
+        return gemm_skinny(x, weight, out_dtype=out_dtype, parts=8 if k >= 16384 else 4, row_tiles=4)
     return linear(x, weight, out_dtype=out_dtype)
+
+
+def deep_or_small(n: int, k: int) -> bool:
+    """Shapes at which, for 17 to 64 rows, the streaming kernel with K cut into parts beats
+    the library product: matrices much deeper than wide (a down projection; the library does
+    not cut K) and small ones (an out projection of a 4B or 8B model).  Measured at 64 rows:
+    2560x4096 14 against 19 us, 2560x9728 25 against 28, 4096x12288 32 against 37,
+    5120x25600 85 against 157; but 5120x8192 34 against 29, which stays with the library."""
+    return k >= 2 * n or n * k <= 24 * 1024 * 1024
 
 
 def linear_glu(x: torch.Tensor, gate_up: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:

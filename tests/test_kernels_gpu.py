@@ -161,6 +161,14 @@ def test_gemm_skinny(ops, shape):
         got = ops.gemm_skinny(a.to(DEV), w.to(DEV), parts=parts)
         assert got.shape == (parts, m, n) and got.dtype == torch.float32
         assert np.abs(f64(got).sum(0) - want).max() <= tol(torch.float32, np.abs(want).max())
+    if m > 16:  # four tiles of w to a workgroup, alone and with K cut
+        for parts in (1, 4, 8):
+            got = ops.gemm_skinny(a.to(DEV), w.to(DEV), out_dtype=torch.float32, parts=parts, row_tiles=4)
+            got = got.sum(0) if parts > 1 else got
+            assert got.shape == (m, n)
+            assert np.abs(f64(got) - want).max() <= tol(torch.float32, np.abs(want).max())
+        one = ops.gemm_skinny(a[5:6].contiguous().to(DEV), w.to(DEV), parts=4)
+        assert torch.equal(one[:, 0], ops.gemm_skinny(a.to(DEV), w.to(DEV), parts=4, row_tiles=4)[:, 5])
     # the same rows give the same bits whatever other rows share the launch
     full = ops.gemm_skinny(a.to(DEV), w.to(DEV), out_dtype=torch.float32)
     alone = ops.gemm_skinny(a[:1].contiguous().to(DEV), w.to(DEV), out_dtype=torch.float32)
