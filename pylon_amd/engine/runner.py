@@ -113,6 +113,7 @@ class Runner:
         runner.config = model_config
         if config.cuda_graphs:
             runner.enable_graphs(config.max_batch_size)
+            runner.capture_graphs()
         return runner
 
     def enable_graphs(self, max_batch: Optional[int] = None, max_tokens_per_request: Optional[int] = None) -> None:
@@ -127,6 +128,37 @@ class Runner:
         self.graphs = DecodeGraphs(self.model, self.manager, self.arena,
                                    max_batch=max_batch or self.manager.slots.max_slots,
                                    max_pages_per_request=-(-limit // page), chosen=self.chosen)
+
+    def capture_graphs(self, batch_sizes: Optional[Seq[int]] = None) -> tuple:
+        """Capture the decode graphs of these batch sizes (default: every size up to the
+        largest the graphs serve) now instead of at their first use, as the reference does
+        at start-up (/root/reference/src/pylon/decode/warmup.py:140-167): throw-away
+        requests of one token each take a decode step per batch size and are closed again.
+        Sizes for which the pool has no free pages or slots are left to their first use.
+        Returns the batch sizes that have a graph."""
+        if self.graphs is None:
+            raise RuntimeError("capture_graphs needs enable_graphs first")
+        from ..cache import OutOfPages
+
+        sizes = sorted(set(batch_sizes or range(1, self.graphs.max_batch + 1)))
+        most = min(max(sizes), self.manager.free_pages, self.manager.slots.free_slots, self.graphs.max_batch)
+        seqs = [self.open(("graph-warm-up", i)) for i in range(most)]
+        try:
+            if seqs:
+                self.step([StepEntry(seq, [0], []) for seq in seqs])
+            for rows in sizes:
+                if rows > most:
+                    break
+                entries = [StepEntry(seq, [0], [0]) for seq in seqs[:rows]]
+                if self.graphs.wants(entries) and (rows, self.graphs._bound(entries)) not in self.graphs.captured:
+                    self.graphs.run(entries)
+        except OutOfPages:
+            pass  # a small pool: the remaining sizes are captured when they first occur
+        finally:
+            for seq in seqs:
+                self.close(seq)
+        self.synchronize()
+        return self.graphs.captured_sizes()
 
     def synchronize(self) -> None:
         torch.cuda.synchronize(self.model.device)

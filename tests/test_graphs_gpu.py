@@ -127,3 +127,37 @@ def test_long_requests_share_their_keys_between_workgroups_in_graphs_too(tmp_pat
         assert np.abs(eager[rid] - want).max() <= 2e-2 * scale, rid
         assert np.abs(graphed[rid] - want).max() <= 2e-2 * scale, rid
         assert np.abs(graphed[rid] - eager[rid]).max() <= 1e-2 * scale, rid
+
+
+def test_graphs_captured_at_start_up(tmp_path):
+    """Every batch size the pool has room for is captured beforehand; later decode steps
+    only replay, with the logits of the same steps run kernel by kernel; the throw-away
+    requests of the capture leave nothing behind."""
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from pylon_amd.engine import Runner, StepEntry
+
+    folder = make_model_folder(tmp_path, "D", dtype="bfloat16", std=0.08)
+    cfg, _ = read_folder(folder)
+    runner = Runner.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=40, max_requests=6)
+    runner.enable_graphs(6)
+    assert runner.capture_graphs() == (1, 2, 3, 4, 5, 6)
+    runner.manager.check()
+    assert runner.manager.free_pages == 40 and not runner.manager.live_sequences()
+    captured = len(runner.graphs.captured)
+    eager = Runner.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=40, max_requests=6)
+    prompts = [random_tokens(cfg["vocab_size"], n, 70 + n) for n in (5, 18, 31)]
+    outs = []
+    for r in (runner, eager):
+        seqs = [r.open(f"s{i}") for i in range(3)]
+        r.step([StepEntry(s, p, []) for s, p in zip(seqs, prompts)])
+        rows = [r.step([StepEntry(s, [7 + t], [0]) for s in seqs[: 3 - t % 2]]).cpu().numpy() for t in range(6)]
+        outs.append(np.concatenate(rows))
+    assert len(runner.graphs.captured) == captured and runner.graphs.replays >= 6 + 6
+    assert np.abs(outs[0] - outs[1]).max() <= 1e-2 * np.abs(outs[1]).max()
+    # a pool too small for the largest sizes: those are left to their first use
+    small = Runner.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=3, max_requests=6)
+    small.enable_graphs(6)
+    assert small.capture_graphs() == (1, 2, 3)
+    small.manager.check()
+    assert small.manager.free_pages == 3
