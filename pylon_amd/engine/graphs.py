@@ -4,9 +4,9 @@ As in the reference (/root/reference/src/pylon/decode/graph.py:71-242) there is 
 per batch size, captured over static buffers; a replay fills the buffers and launches the
 graph; a batch size without a graph, or whose capture failed, runs kernel by kernel, and a
 failed capture is not tried again.  Differences: the static buffers are one packed block
-of metadata (filled by the same code that prepares any other step), graphs are captured
-the first time a batch size is seen rather than all at start-up, and a batch is never
-padded to a larger captured size.
+of metadata (filled by the same code that prepares any other step), a graph that was not
+captured at start-up (``Runner.capture_graphs``) is captured the first time its batch size
+is seen, and a batch is never padded to a larger captured size.
 
 The launches recorded in a graph must not depend on the requests' lengths: the block
 table has a fixed width, and how the decode attention kernel shares a request's keys
