@@ -353,8 +353,9 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   store_tile<HD, QT>(out, o, wave, col, grp, group, tok0, ntok, n_heads, kvh * group);
 }
 
-// The same for head size 128 and pages that are powers of two of at least 64, with the two
-// matrix-instruction-era features of this chip that take the copying out of the loop:
+// The same for head size 128 and pages that are powers of two of at least 64, with two
+// instructions of gfx950 that take the copying out of the loop (global_load_lds_dwordx4 and
+// ds_read_b64_tr_b16):
 //
 //  * Keys and values go from the cache straight into LDS (16 bytes per lane, a wave fills
 //    1 KB of consecutive LDS from 64 places of its choice), two buffers each, so that the
