@@ -64,8 +64,10 @@ __device__ __forceinline__ void store4(bf16_t* p, long long c, float a, float b,
 // One workgroup per output row. `row_idx` (optional) picks the input row of each
 // output row. With `delta`, the input is resid + delta (float sum); `write_resid`
 // stores that sum back into resid (only meaningful without row_idx).
+// At most 512 threads per workgroup, so that a thread may hold the eight partial sums of its
+// sixteen elements in registers (a kernel that may be launched with 1,024 threads gets 128).
 template <typename TX, typename TD, typename TO>
-__global__ void rmsnorm_kernel(TO* __restrict__ out, TX* x, const TD* __restrict__ delta,
+__global__ __launch_bounds__(512) void rmsnorm_kernel(TO* __restrict__ out, TX* x, const TD* __restrict__ delta,
                                int n_delta, long long delta_stride,
                                const float* __restrict__ w, const int* __restrict__ row_idx,
                                int dim, float eps, int write_resid) {
@@ -186,7 +188,7 @@ template <typename TX, typename TD>
 static void launch_rmsnorm_out(void* out, int out_dtype, TX* x, const TD* delta, int n_delta,
                                long long delta_stride, const float* w, const int* row_idx, int rows,
                                int dim, float eps, int write_resid, hipStream_t stream) {
-  dim3 grid(rows), block(dim > 4096 ? 1024 : 256);
+  dim3 grid(rows), block(dim > 4096 ? 512 : 256);
   if (out_dtype == PYLON_F32)
     hipLaunchKernelGGL((rmsnorm_kernel<TX, TD, float>), grid, block, 0, stream, (float*)out, x, delta,
                        n_delta, delta_stride, w, row_idx, dim, eps, write_resid);

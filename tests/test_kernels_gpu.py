@@ -147,6 +147,38 @@ def test_gemm_rows_do_not_depend_on_the_batch(ops):
         assert torch.equal(part, whole[lo:hi])
 
 
+@pytest.mark.parametrize("dim", [80, 2560 + 16, 5120 + 8, 9000])
+@pytest.mark.parametrize("parts", [1, 2, 3, 4, 8])
+def test_residual_norm_adds_partial_sums(ops, dim, parts):
+    """A stack of float partial sums of a matrix product (K cut in parts) is added to the
+    residual in a fixed order and normed: rows of every width class of the kernel (one that
+    fits 256 threads' registers, one that needs 512, one that takes the general loop)."""
+    eps, rows = 2e-6, 5
+    x = rnd((rows, dim), 12, torch.float32, 2.0)
+    stack = rnd((parts, rows, dim), 13, torch.float32)
+    w = 1 + 0.3 * rnd((dim,), 14)
+    summed = f64(x) + f64(stack).sum(0)
+    want = summed / np.sqrt((summed * summed).mean(-1, keepdims=True) + eps) * f64(w)
+    for out_dtype in (torch.bfloat16, torch.float32):
+        resid = x.clone().to(DEV)
+        got = ops.add_rmsnorm(resid, stack.to(DEV), w.to(DEV), eps, out_dtype)
+        assert np.abs(f64(resid) - summed).max() <= 1e-6 * np.abs(summed).max()
+        assert np.abs(f64(got) - want).max() <= tol(out_dtype, np.abs(want).max())
+    # the same bits as adding the parts one after the other in float32
+    resid = x.clone().to(DEV)
+    ops.add_rmsnorm(resid, stack.to(DEV), w.to(DEV), eps, torch.float32)
+    one_by_one = stack[0].clone()
+    for p in range(1, parts):
+        one_by_one += stack[p]
+    assert torch.equal(resid.cpu(), x + one_by_one)
+    # picked rows: the residual stays
+    resid = x.clone().to(DEV)
+    idx = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
+    got = ops.add_rmsnorm(resid, stack.to(DEV), w.to(DEV), eps, torch.float32, row_idx=idx)
+    assert torch.equal(resid.cpu(), x)
+    assert np.abs(f64(got) - want[[4, 1]]).max() <= tol(torch.float32, np.abs(want).max())
+
+
 @pytest.mark.parametrize("shape", [(1, 96, 80), (8, 301, 176), (16, 130, 1000), (17, 64, 64),
                                    (64, 2560 + 8, 512 + 24), (33, 48, 4096), (8, 72, 9728)])
 def test_gemm_skinny(ops, shape):
