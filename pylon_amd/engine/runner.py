@@ -146,8 +146,9 @@ class Runner:
         try:
             if seqs:
                 self.step([StepEntry(seq, [0], []) for seq in seqs])
+            limit = self.model.spec.max_positions
             for rows in sizes:
-                if rows > most:
+                if rows > most or (limit and seqs[0].length + 1 > limit):
                     break
                 entries = [StepEntry(seq, [0], [0]) for seq in seqs[:rows]]
                 if self.graphs.wants(entries) and (rows, self.graphs._bound(entries)) not in self.graphs.captured:
