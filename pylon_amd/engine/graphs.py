@@ -56,6 +56,15 @@ class DecodeGraphs:
             bound *= 2
         return bound
 
+    def bounds(self) -> Tuple[int, ...]:
+        """Every bound a graph may be captured for: the powers of two from 1024 up to the one
+        that holds the longest request the block table has room for."""
+        longest = self.width * self.manager.page_size
+        out = [1024]
+        while out[-1] < longest:
+            out.append(out[-1] * 2)
+        return tuple(out)
+
     def wants(self, entries: Seq[StepEntry]) -> bool:
         """A decode-only step: one token per request, each wanting its logits."""
         rows = len(entries)
@@ -69,14 +78,16 @@ class DecodeGraphs:
                 return False  # longer than the captured block table: run kernel by kernel
         return True
 
-    def run(self, entries: Seq[StepEntry]) -> Optional[torch.Tensor]:
+    def run(self, entries: Seq[StepEntry], bound: Optional[int] = None) -> Optional[torch.Tensor]:
         """Replay (capturing first if need be).  Returns None if this batch size has no
         graph; the caller then runs the step kernel by kernel.  The cache is reserved and
-        committed here exactly as an ordinary step does."""
+        committed here exactly as an ordinary step does.  ``bound`` (capture at start-up)
+        asks for the graph of a larger bound than these requests need: what a graph records
+        depends on the bound, not on the lengths, so short requests can capture it."""
         rows = len(entries)
         manager, model, arena = self.manager, self.model, self.arena
         pairs = [(e.seq, 1) for e in entries]
-        bound = self._bound(entries)
+        bound = max(bound or 0, self._bound(entries))
         key = (rows, bound)
         entry = self.captured.get(key)
         if entry is None:

@@ -129,32 +129,35 @@ class Runner:
                                    max_batch=max_batch or self.manager.slots.max_slots,
                                    max_pages_per_request=-(-limit // page), chosen=self.chosen)
 
-    def capture_graphs(self, batch_sizes: Optional[Seq[int]] = None) -> tuple:
-        """Capture the decode graphs of these batch sizes (default: every size up to the
-        largest the graphs serve) now instead of at their first use, as the reference does
-        at start-up (/root/reference/src/pylon/decode/warmup.py:140-167): throw-away
-        requests of one token each take a decode step per batch size and are closed again.
-        Sizes for which the pool has no free pages or slots are left to their first use.
-        Returns the batch sizes that have a graph."""
+    def capture_graphs(self, batch_sizes: Optional[Seq[int]] = None, bounds: Optional[Seq[int]] = None) -> tuple:
+        """Capture decode graphs now instead of at their first use, as the reference does at
+        start-up (/root/reference/src/pylon/decode/warmup.py:140-167): for these batch sizes
+        (default: every size the graphs serve) and these bounds on the requests' lengths
+        (default: every bound, see :meth:`DecodeGraphs.bounds`).  Throw-away requests of one
+        token each take one decode step per graph and are closed again.  Sizes for which the
+        pool has no free pages or slots are left to their first use.  Returns the batch sizes
+        that have a graph."""
         if self.graphs is None:
             raise RuntimeError("capture_graphs needs enable_graphs first")
         from ..cache import OutOfPages
 
         sizes = sorted(set(batch_sizes or range(1, self.graphs.max_batch + 1)))
+        bounds = sorted(set(bounds or self.graphs.bounds()))
         most = min(max(sizes), self.manager.free_pages, self.manager.slots.free_slots, self.graphs.max_batch)
         seqs = [self.open(("graph-warm-up", i)) for i in range(most)]
+        limit = self.model.spec.max_positions
         try:
             if seqs:
                 self.step([StepEntry(seq, [0], []) for seq in seqs])
-            limit = self.model.spec.max_positions
-            for rows in sizes:
-                if rows > most or (limit and seqs[0].length + 1 > limit):
-                    break
-                entries = [StepEntry(seq, [0], [0]) for seq in seqs[:rows]]
-                if self.graphs.wants(entries) and (rows, self.graphs._bound(entries)) not in self.graphs.captured:
-                    self.graphs.run(entries)
+            for bound in bounds:
+                for rows in sizes:
+                    if rows > most or (limit and seqs[0].length + 1 > limit):
+                        break
+                    entries = [StepEntry(seq, [0], [0]) for seq in seqs[:rows]]
+                    if self.graphs.wants(entries) and (rows, bound) not in self.graphs.captured:
+                        self.graphs.run(entries, bound=bound)
         except OutOfPages:
-            pass  # a small pool: the remaining sizes are captured when they first occur
+            pass  # a small pool: the remaining graphs are captured when they first occur
         finally:
             for seq in seqs:
                 self.close(seq)

@@ -161,3 +161,18 @@ def test_graphs_captured_at_start_up(tmp_path):
     assert small.capture_graphs() == (1, 2, 3)
     small.manager.check()
     assert small.manager.free_pages == 3
+    # every bound on the lengths is captured too, by short requests; a long request then only replays
+    big = Runner.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=140, max_requests=3)
+    big.enable_graphs(2)
+    assert big.graphs.bounds() == (1024, 2048, 4096)
+    big.capture_graphs()
+    assert set(big.graphs.captured) == {(rows, bound) for rows in (1, 2) for bound in (1024, 2048, 4096)}
+    plain_runner = Runner.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=140, max_requests=3)
+    long_prompt = random_tokens(cfg["vocab_size"], 1100, 5)
+    outs = []
+    for r in (big, plain_runner):
+        seq = r.open("long")
+        r.step([StepEntry(seq, long_prompt, [])])
+        outs.append(np.concatenate([r.step([StepEntry(seq, [11 + t], [0])]).cpu().numpy() for t in range(4)]))
+    assert len(big.graphs.captured) == 6 and big.graphs.replays >= 6 + 4
+    assert np.abs(outs[0] - outs[1]).max() <= 1e-2 * np.abs(outs[1]).max()
