@@ -1,0 +1,90 @@
+"""The layer sizes the benchmark runs (Qwen3-4B: width 2560, 32 query and 8 key/value heads of
+128, feed-forward 9728, pages of 256 tokens), with two layers and a small vocabulary so that
+the plain implementation stays quick: the kernels chosen at these sizes (the attention kernel
+that loads pages straight into LDS, the weight-streaming products with K cut in parts, the
+fused decode attention, decode graphs) against the plain model, whole and cut."""
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import make_model_folder, random_tokens, read_folder
+from tests.plain import qwen3 as plain
+
+pytestmark = pytest.mark.gpu
+
+REAL = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_act="silu", attention_bias=False,
+    num_hidden_layers=2, hidden_size=2560, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+    intermediate_size=9728, vocab_size=2048, rope_theta=5000000.0, rms_norm_eps=1e-6,
+    tie_word_embeddings=True, max_position_embeddings=8192,
+)
+
+
+@pytest.fixture(scope="module")
+def real(tmp_path_factory):
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    folder = make_model_folder(tmp_path_factory.mktemp("real"), "real", dtype="bfloat16", config=REAL,
+                               seed=3, norm_jitter=0.1)
+    cfg, weights = read_folder(folder)
+    prompts = [random_tokens(cfg["vocab_size"], n, 900 + n) for n in (300, 70, 17)]
+    want = [plain.forward(weights, cfg, p) for p in prompts]
+    return folder, cfg, prompts, want
+
+
+@pytest.mark.parametrize("dtype,bound", [("float32", 2e-5), ("bfloat16", 3e-2)])
+def test_benchmark_layer_sizes_match_the_plain_model(real, dtype, bound):
+    from pylon_amd.engine import Runner, StepEntry
+
+    folder, cfg, prompts, want = real
+    runner = Runner.from_folder(folder, dtype=dtype, page_size=256, num_pages=8, max_requests=4)
+    runner.enable_graphs(4)
+    seqs = [runner.open(f"r{i}") for i in range(3)]
+    # the first 270, 45 and 9 tokens as prompt portions of one step, the rest decoded one by one
+    # (the three requests side by side while they last: batches of 3, 2 and 1, from graphs)
+    heads = (270, 45, 9)
+    got = [[] for _ in prompts]
+    out = runner.step([StepEntry(s, p[:h], list(range(h))) for s, p, h in zip(seqs, prompts, heads)]).cpu().numpy()
+    at = 0
+    for i, h in enumerate(heads):
+        got[i].append(out[at: at + h])
+        at += h
+    for t in range(30):
+        live = [i for i in range(3) if heads[i] + t < len(prompts[i])]
+        if not live:
+            break
+        out = runner.step([StepEntry(seqs[i], [prompts[i][heads[i] + t]], [0]) for i in live]).cpu().numpy()
+        for row, i in enumerate(live):
+            got[i].append(out[row: row + 1])
+    assert runner.graphs.replays >= 20 and set(runner.graphs.captured_sizes()) == {1, 2, 3}
+    for i, ref in enumerate(want):
+        g = np.concatenate(got[i])
+        scale = np.abs(ref).max()
+        err = np.abs(g - ref[: len(g)]).max(axis=1)
+        assert err.max() <= bound * scale, (dtype, i, int(err.argmax()), float(err.max()), float(scale))
+
+
+@pytest.mark.parametrize("dtype,bound", [("float32", 2e-5), ("bfloat16", 3e-2)])
+def test_twenty_requests_decode_side_by_side(real, dtype, bound):
+    """Batches of 17 to 64 rows: the out and down projections run on the streaming kernel with
+    64 weight rows per workgroup, the other products in the library."""
+    from pylon_amd.engine import Runner, StepEntry
+
+    folder, cfg, _, _ = real
+    _, weights = read_folder(folder)
+    requests = [random_tokens(cfg["vocab_size"], 9 + i, 700 + i) for i in range(20)]
+    want = [plain.forward(weights, cfg, r) for r in requests]
+    runner = Runner.from_folder(folder, dtype=dtype, page_size=256, num_pages=20, max_requests=20)
+    runner.enable_graphs(20)
+    seqs = [runner.open(f"q{i}") for i in range(20)]
+    decoded = 5
+    runner.step([StepEntry(s, r[:-decoded], []) for s, r in zip(seqs, requests)])
+    rows = []
+    for t in range(decoded):
+        entries = [StepEntry(s, [r[len(r) - decoded + t]], [0]) for s, r in zip(seqs, requests)]
+        rows.append(runner.step(entries).cpu().numpy())
+    assert runner.graphs.captured_sizes() == (20,) and runner.graphs.replays == decoded
+    for i, ref in enumerate(want):
+        got = np.stack([rows[t][i] for t in range(decoded)])
+        scale = np.abs(ref).max()
+        assert np.abs(got - ref[-decoded:]).max() <= bound * scale, (dtype, i)
