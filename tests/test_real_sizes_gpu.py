@@ -88,3 +88,35 @@ def test_twenty_requests_decode_side_by_side(real, dtype, bound):
         got = np.stack([rows[t][i] for t in range(decoded)])
         scale = np.abs(ref).max()
         assert np.abs(got - ref[-decoded:]).max() <= bound * scale, (dtype, i)
+
+
+WIDE = dict(REAL, num_hidden_layers=1, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8,
+            intermediate_size=16384, vocab_size=1024, rope_theta=1000000.0, tie_word_embeddings=False)
+
+
+def test_a_layer_of_the_widest_shape(tmp_path):
+    """Width 5120 with 64 query heads over 8 key/value heads, as Qwen3-32B (the feed-forward
+    narrower, to keep the plain model quick, but deep enough that the down projection's K is
+    cut in eight): the norm's wide rows, groups of eight heads in decode attention, and the
+    eight partial sums, for a prompt portion and for 20 requests decoding side by side."""
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from pylon_amd.engine import Runner, StepEntry
+
+    folder = make_model_folder(tmp_path, "wide", dtype="bfloat16", config=WIDE, seed=4, norm_jitter=0.1)
+    cfg, weights = read_folder(folder)
+    requests = [random_tokens(cfg["vocab_size"], 6 + 3 * i, 800 + i) for i in range(20)]
+    want = [plain.forward(weights, cfg, r) for r in requests]
+    runner = Runner.from_folder(folder, dtype="bfloat16", page_size=256, num_pages=20, max_requests=20)
+    seqs = [runner.open(f"w{i}") for i in range(20)]
+    decoded = 3
+    first = runner.step([StepEntry(s, r[:-decoded], list(range(len(r) - decoded)))
+                         for s, r in zip(seqs, requests)]).cpu().numpy()
+    rows = [runner.step([StepEntry(s, [r[len(r) - decoded + t]], [0]) for s, r in zip(seqs, requests)]).cpu().numpy()
+            for t in range(decoded)]
+    at = 0
+    for i, ref in enumerate(want):
+        n = len(requests[i]) - decoded
+        got = np.concatenate([first[at: at + n], np.stack([rows[t][i] for t in range(decoded)])])
+        at += n
+        assert np.abs(got - ref).max() <= 3e-2 * np.abs(ref).max(), i
