@@ -40,27 +40,33 @@ def test_benchmark_layer_sizes_match_the_plain_model(real, dtype, bound):
     runner = Runner.from_folder(folder, dtype=dtype, page_size=256, num_pages=8, max_requests=4)
     runner.enable_graphs(4)
     seqs = [runner.open(f"r{i}") for i in range(3)]
-    # the first 270, 45 and 9 tokens as prompt portions of one step, the rest decoded one by one
-    # (the three requests side by side while they last: batches of 3, 2 and 1, from graphs)
-    heads = (270, 45, 9)
+    # the first 270, 45 and 9 tokens as prompt portions of one step; then a mixed step (one
+    # token of two requests beside ten tokens of the third); the rest decoded one by one, the
+    # three requests side by side while they last: batches of 3, 2 and 1, from graphs
+    cursor = [0, 0, 0]
     got = [[] for _ in prompts]
-    out = runner.step([StepEntry(s, p[:h], list(range(h))) for s, p, h in zip(seqs, prompts, heads)]).cpu().numpy()
-    at = 0
-    for i, h in enumerate(heads):
-        got[i].append(out[at: at + h])
-        at += h
-    for t in range(30):
-        live = [i for i in range(3) if heads[i] + t < len(prompts[i])]
-        if not live:
-            break
-        out = runner.step([StepEntry(seqs[i], [prompts[i][heads[i] + t]], [0]) for i in live]).cpu().numpy()
-        for row, i in enumerate(live):
-            got[i].append(out[row: row + 1])
+
+    def run(counts):
+        live = [i for i in range(3) if counts[i]]
+        entries = [StepEntry(seqs[i], prompts[i][cursor[i]: cursor[i] + counts[i]], list(range(counts[i])))
+                   for i in live]
+        out = runner.step(entries).cpu().numpy()
+        at = 0
+        for i in live:
+            got[i].append(out[at: at + counts[i]])
+            at += counts[i]
+            cursor[i] += counts[i]
+
+    run([270, 45, 9])
+    run([1, 10, 1])
+    while any(cursor[i] < len(prompts[i]) for i in range(3)):
+        run([1 if cursor[i] < len(prompts[i]) else 0 for i in range(3)])
     assert runner.graphs.replays >= 20 and set(runner.graphs.captured_sizes()) == {1, 2, 3}
     for i, ref in enumerate(want):
         g = np.concatenate(got[i])
         scale = np.abs(ref).max()
-        err = np.abs(g - ref[: len(g)]).max(axis=1)
+        assert len(g) == len(ref)
+        err = np.abs(g - ref).max(axis=1)
         assert err.max() <= bound * scale, (dtype, i, int(err.argmax()), float(err.max()), float(scale))
 
 
