@@ -226,11 +226,12 @@ def mixed_run(runner, cfg, batch: int, prompt_len: int, repeats: int, seed: int)
     return times[len(times) // 2]
 
 
-def engine_run(runner, cfg, batch: int, seed: int, prompt_len: int = PROMPT_LEN, new_tokens: int = NEW_TOKENS) -> float:
+def engine_run(runner, cfg, batch: int, seed: int, prompt_len: int = PROMPT_LEN, new_tokens: int = NEW_TOKENS):
     """The same work through the scheduler: ``batch`` requests of ``prompt_len`` random ids and
     ``new_tokens`` greedy tokens each, queued at once; generated tokens per second from the
     first request's arrival to the last one's end (admission, the prompts' prefill, ticks,
-    sampling and the host's reading of every token included)."""
+    sampling and the host's reading of every token included), and the median time from a
+    request's arrival to its first token in milliseconds."""
     import numpy as np
     import torch
 
@@ -249,7 +250,8 @@ def engine_run(runner, cfg, batch: int, seed: int, prompt_len: int = PROMPT_LEN,
     results = engine.generate(prompts, sampling)
     elapsed = time.perf_counter() - started
     assert all(len(r.output_ids) == new_tokens for r in results)
-    return batch * new_tokens / elapsed
+    first = sorted(r.first_token_seconds for r in results)
+    return batch * new_tokens / elapsed, 1e3 * first[len(first) // 2]
 
 
 def main() -> int:
@@ -346,11 +348,13 @@ def main() -> int:
             n = min(steps, 256)
             e, _ = decode_run(runner, cfg, batch, n, args.warmup, seed=3 + batch, prompt_len=prompt_len)
             points[f"decode_b{batch}"] = round(batch * n / e, 1)
-        points["engine_b8"] = round(engine_run(runner, cfg, batch=8, seed=9, prompt_len=prompt_len), 1)
+        rate, first_ms = engine_run(runner, cfg, batch=8, seed=9, prompt_len=prompt_len)
+        points["engine_b8"], points["engine_b8_first_token_ms"] = round(rate, 1), round(first_ms, 2)
         # the reference's other published workload: 2,048-token prompts, 32 new tokens, 8 at a time
-        # (53.7 output tokens/s on its L4, /root/reference/README.md:76)
-        points["engine_prefill_heavy_b8"] = round(
-            engine_run(runner, cfg, batch=8, seed=10, prompt_len=PREFILL_TOKENS, new_tokens=32), 1)
+        # (53.7 output tokens/s and 847 ms to the first token on its L4, /root/reference/README.md:76,90)
+        rate, first_ms = engine_run(runner, cfg, batch=8, seed=10, prompt_len=PREFILL_TOKENS, new_tokens=32)
+        points["engine_prefill_heavy_b8"] = round(rate, 1)
+        points["engine_prefill_heavy_b8_first_token_ms"] = round(first_ms, 2)
         record["points"] = points
     print(json.dumps(record))
     return 0
