@@ -70,12 +70,13 @@ def build_runner(shape: dict, layers: int, dtype: str, max_requests: int, num_pa
 
     from pylon_amd.config import resolve
     from pylon_amd.engine import Model, Runner, resolve_dtype
+    from pylon_amd.weights import fill_random_model
 
     raw = config_json(shape, layers)
     arch = resolve(raw)
     cfg = arch.parse_config(raw)
     model = Model(arch.model_spec(cfg), dtype=resolve_dtype(dtype), device="cuda:0")
-    model.init_random(seed=0)
+    fill_random_model(model, arch, cfg, seed=0, std=0.02)  # the random-weights mode, on the device
     runner = Runner(model, page_size=PAGE_SIZE, num_pages=num_pages, max_requests=max_requests)
     if graphs:
         runner.enable_graphs(max_requests, max_tokens_per_request=shape["max_position_embeddings"])
@@ -103,25 +104,25 @@ def linear_flops_per_token(cfg) -> float:
 
 
 def feed_prompts(runner, sampler, seqs, prompts) -> None:
-    """The prompts through the step function in steps of at most PREFILL_TOKENS tokens, cut as
-    the scheduler cuts them (short prompts side by side, a long one in portions); the first
-    new token of each request is chosen on the device."""
+    """The prompts through the step function in steps of at most PREFILL_TOKENS tokens, cut by
+    the scheduler's own rule (:func:`pylon_amd.engine.scheduler.cut_prompts`: short prompts
+    side by side, a long one in portions); the first new token of each request is chosen on
+    the device."""
     from pylon_amd.engine import StepEntry
+    from pylon_amd.engine.scheduler import PromptWork, cut_prompts
     from pylon_amd.sampling import Sampling
 
     fed = [0] * len(seqs)
-    at = 0
-    while at < len(seqs):
-        entries, budget = [], PREFILL_TOKENS
-        while at < len(seqs) and budget > 0:
-            take = min(budget, len(prompts[at]) - fed[at])
-            last = fed[at] + take == len(prompts[at])
-            entries.append(StepEntry(seqs[at], prompts[at][fed[at]: fed[at] + take], [take - 1] if last else []))
-            fed[at] += take
-            budget -= take
-            if not last:
-                break
-            at += 1
+    while True:
+        work = [PromptWork(i, len(prompts[i]) - fed[i], 0.0) for i in range(len(seqs)) if fed[i] < len(prompts[i])]
+        portions = cut_prompts(work, PREFILL_TOKENS, 0.0)
+        if not portions:
+            return
+        entries = []
+        for i, take in portions:
+            last = fed[i] + take == len(prompts[i])
+            entries.append(StepEntry(seqs[i], prompts[i][fed[i]: fed[i] + take], [take - 1] if last else []))
+            fed[i] += take
         out = runner.step(entries)
         wanted = sum(len(e.want) for e in entries)
         if wanted:

@@ -202,64 +202,69 @@ def build_step(entries: Seq[StepEntry], manager: CacheManager, arena: MetadataAr
     pairs = [(e.seq, int(c)) for e, c in zip(entries, counts)]
     manager.reserve(pairs)  # all-or-nothing
 
-    starts = np.fromiter((e.seq.length for e in entries), dtype=np.int64, count=rows)
-    slots = np.fromiter((e.seq.slot for e in entries), dtype=np.int64, count=rows)
-    tok_row = np.repeat(np.arange(rows, dtype=np.int64), counts)
-    positions = starts[tok_row] + (np.arange(tokens, dtype=np.int64) - row_start[tok_row])
-    seq_lens = starts + counts
-    need_width = int(-(-seq_lens.max() // manager.page_size))
-    if width is None:
-        width = need_width
-    elif need_width > width:
+    # From here on pages are held for this step: whatever goes wrong before the step's
+    # metadata is on the device gives them back.
+    try:
+        starts = np.fromiter((e.seq.length for e in entries), dtype=np.int64, count=rows)
+        slots = np.fromiter((e.seq.slot for e in entries), dtype=np.int64, count=rows)
+        tok_row = np.repeat(np.arange(rows, dtype=np.int64), counts)
+        positions = starts[tok_row] + (np.arange(tokens, dtype=np.int64) - row_start[tok_row])
+        seq_lens = starts + counts
+        need_width = int(-(-seq_lens.max() // manager.page_size))
+        if width is None:
+            width = need_width
+        elif need_width > width:
+            raise ValueError(f"a request needs {need_width} pages but the block table holds {width}")
+
+        n_groups = len(manager.groups)
+        layout, size = plan_layout(tokens, rows, len(logit_list), n_groups, width)
+        host, index = arena.acquire(size)
+
+        def seg(name: str) -> np.ndarray:
+            off, n = layout[name]
+            return host[off: off + n]
+
+        token_slots = slots[tok_row]
+        if pending.any():
+            flat = np.where(pending, -1 - token_slots, flat)  # the embedding reads chosen[slot]
+        seg("token_ids")[:] = flat
+        seg("positions")[:] = positions
+        seg("tok_row")[:] = tok_row
+        seg("row_start")[:] = row_start
+        seg("seq_lens")[:] = seq_lens
+        seg("row_slots")[:] = slots
+        seg("row_first")[:] = starts == 0
+        if logit_list:
+            seg("logit_idx")[:] = logit_list
+            seg("logit_slots")[:] = token_slots[logit_list]
+        for g in range(n_groups):
+            manager.slot_map(g, token_slots, positions, seg(f"slot_map{g}"))
+            manager.block_table(g, slots, width, seg(f"block_table{g}").reshape(rows, width))
+        block = arena.upload(index, size, into=device_block)
+
+        def dev(name: str) -> torch.Tensor:
+            off, n = layout[name]
+            return block[off: off + n]
+
+        views: Dict[int, CacheView] = {}
+        for cache_id in range(manager.n_caches):
+            view = manager.view(cache_id)
+            if view.group >= 0:
+                view.slot_map = dev(f"slot_map{view.group}")
+                view.block_table = dev(f"block_table{view.group}").view(rows, width)
+            views[cache_id] = view
+        return StepContext(
+            tokens=tokens, rows=rows,
+            token_ids=dev("token_ids"), positions=dev("positions"), tok_row=dev("tok_row"),
+            row_start=dev("row_start"), seq_lens=dev("seq_lens"), row_slots=dev("row_slots"),
+            row_first=dev("row_first"),
+            logit_idx=dev("logit_idx") if logit_list else None, n_logits=len(logit_list),
+            logit_slots=dev("logit_slots") if logit_list else None, chosen=chosen,
+            views=views, counts=counts, starts=starts, max_count=int(counts.max()),
+            max_len=int(seq_lens.max()) if len_bound is None else int(len_bound),
+            decode_only=bool((counts == 1).all()),
+            fixed_shapes=fixed_shapes,
+        )
+    except BaseException:
         manager.cancel(pairs)
-        raise ValueError(f"a request needs {need_width} pages but the block table holds {width}")
-
-    n_groups = len(manager.groups)
-    layout, size = plan_layout(tokens, rows, len(logit_list), n_groups, width)
-    host, index = arena.acquire(size)
-
-    def seg(name: str) -> np.ndarray:
-        off, n = layout[name]
-        return host[off: off + n]
-
-    token_slots = slots[tok_row]
-    if pending.any():
-        flat = np.where(pending, -1 - token_slots, flat)  # the embedding reads chosen[slot]
-    seg("token_ids")[:] = flat
-    seg("positions")[:] = positions
-    seg("tok_row")[:] = tok_row
-    seg("row_start")[:] = row_start
-    seg("seq_lens")[:] = seq_lens
-    seg("row_slots")[:] = slots
-    seg("row_first")[:] = starts == 0
-    if logit_list:
-        seg("logit_idx")[:] = logit_list
-        seg("logit_slots")[:] = token_slots[logit_list]
-    for g in range(n_groups):
-        manager.slot_map(g, token_slots, positions, seg(f"slot_map{g}"))
-        manager.block_table(g, slots, width, seg(f"block_table{g}").reshape(rows, width))
-    block = arena.upload(index, size, into=device_block)
-
-    def dev(name: str) -> torch.Tensor:
-        off, n = layout[name]
-        return block[off: off + n]
-
-    views: Dict[int, CacheView] = {}
-    for cache_id in range(manager.n_caches):
-        view = manager.view(cache_id)
-        if view.group >= 0:
-            view.slot_map = dev(f"slot_map{view.group}")
-            view.block_table = dev(f"block_table{view.group}").view(rows, width)
-        views[cache_id] = view
-    return StepContext(
-        tokens=tokens, rows=rows,
-        token_ids=dev("token_ids"), positions=dev("positions"), tok_row=dev("tok_row"),
-        row_start=dev("row_start"), seq_lens=dev("seq_lens"), row_slots=dev("row_slots"),
-        row_first=dev("row_first"),
-        logit_idx=dev("logit_idx") if logit_list else None, n_logits=len(logit_list),
-        logit_slots=dev("logit_slots") if logit_list else None, chosen=chosen,
-        views=views, counts=counts, starts=starts, max_count=int(counts.max()),
-        max_len=int(seq_lens.max()) if len_bound is None else int(len_bound),
-        decode_only=bool((counts == 1).all()),
-        fixed_shapes=fixed_shapes,
-    )
+        raise

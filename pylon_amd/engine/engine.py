@@ -17,7 +17,9 @@ token is dropped.  The end by ``max_new_tokens`` is known beforehand and costs n
 """
 from __future__ import annotations
 
+import dataclasses
 import logging
+import random
 import threading
 import time
 from collections import deque
@@ -51,7 +53,9 @@ class GenerationResult:
     prefill_seconds: float
     inter_token_seconds: List[float]
     queue_seconds: float
+    first_token_at: Optional[float] = None  # on the engine's clock
     first_token_seconds: Optional[float] = None
+    token_intervals: Optional[Tuple[float, ...]] = None  # between the reads of emitted tokens
     elapsed_seconds: Optional[float] = None
 
 
@@ -98,6 +102,8 @@ class Active:
     inter_token_seconds: List[float] = field(default_factory=list)
     prompt_wait_started: float = 0.0
     first_token_at: Optional[float] = None
+    last_token_at: Optional[float] = None
+    token_intervals: List[float] = field(default_factory=list)
     # Running ahead: a sampled token waits on the device to be fed / how many sampled
     # tokens the host has not read yet / the request has ended.
     awaiting: bool = False
@@ -161,6 +167,7 @@ class Engine:
         self._closed = False
         self.head_skips = 0
         self._serial = 0
+        self._seeds = random.Random()  # seeds of requests that bring none (from the system's entropy)
         self.steps_run = 0
         self.last_step = None  # (decode rows, prompt portions) of the most recent step
         self._thread: Optional[threading.Thread] = None
@@ -193,6 +200,11 @@ class Engine:
     def enqueue(self, input_ids: Sequence[int], eos_token_id=None, sampling: Optional[Sampling] = None,
                 request_id: Optional[str] = None) -> Future:
         sampling = sampling or Sampling()
+        if sampling.seed is None:
+            # No seed given: every request draws from a stream of its own, as requests of
+            # the reference differ, which all draw from one global generator
+            # (/root/reference/src/pylon/decode/runner.py:513-525).  A given seed repeats.
+            sampling = dataclasses.replace(sampling, seed=self._seeds.getrandbits(63))
         request_id = request_id or "internal"
         stop_ids = _stop_ids(eos_token_id)
         input_ids = list(input_ids)
@@ -424,6 +436,9 @@ class Engine:
         if token_id in item.request.stop_ids:
             self._complete(item, "eos")
             return False
+        if item.last_token_at is not None:
+            item.token_intervals.append(sampled_at - item.last_token_at)
+        item.last_token_at = sampled_at
         item.output_ids.append(token_id)
         if len(item.output_ids) == item.request.sampling.max_new_tokens:
             self._complete(item, "length")
@@ -438,7 +453,9 @@ class Engine:
         result = GenerationResult(
             output_ids=item.output_ids, finish_reason=reason, prefill_seconds=item.prefill_seconds,
             inter_token_seconds=item.inter_token_seconds, queue_seconds=item.queue_seconds,
+            first_token_at=item.first_token_at,
             first_token_seconds=None if item.first_token_at is None else item.first_token_at - arrived,
+            token_intervals=tuple(item.token_intervals),
             elapsed_seconds=self._clock() - arrived,
         )
         if not item.ticket.future.done():

@@ -116,13 +116,21 @@ class DecodeGraphs:
                     gc.enable()
             self.captured[key] = (graph, block, logits, ctx.logit_slots)
             self.last_logit_slots = ctx.logit_slots
-            graph.replay()  # capture records only; this runs the step
+            try:
+                graph.replay()  # capture records only; this runs the step
+            except BaseException:
+                manager.cancel(pairs)
+                raise
         else:
             graph, block, logits, self.last_logit_slots = entry
             build_step(entries, manager, arena, vocab_size=model.spec.vocab_size,
                        width=self.width, device_block=block, fixed_shapes=True, chosen=self.chosen,
                        len_bound=bound)
-            graph.replay()
+            try:
+                graph.replay()
+            except BaseException:
+                manager.cancel(pairs)  # the pages taken for this step go back
+                raise
         self.replays += 1
         manager.commit(pairs)
         return logits

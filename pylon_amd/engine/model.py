@@ -71,20 +71,3 @@ class Model(Part):
             return None
         h = self.final_norm.add_forward(resid, delta, row_idx=ctx.logit_idx)
         return ops.linear(h, self.head_weight, out_dtype=torch.float32)
-
-    # ---- random weights in place (for measurements at sizes not worth writing to disk) ----
-    def init_random(self, seed: int, std: float = 0.02) -> None:
-        gen = torch.Generator(device=self.device)
-        gen.manual_seed(seed)
-        for path, owner, name in self.named_params():
-            tensor = owner.params[name]
-            if owner.param_roles[name] == "vector":
-                tensor.fill_(1.0)
-            else:
-                # Drawn in slabs so that no float32 copy of a large matrix is needed.
-                flat = tensor.view(-1)
-                step = 1 << 26
-                for start in range(0, flat.numel(), step):
-                    part = flat[start: start + step]
-                    part.copy_(torch.randn(part.numel(), generator=gen, device=self.device,
-                                           dtype=torch.float32) * std)

@@ -489,13 +489,32 @@ def k_parts(n: int, k: int) -> int:
     return parts
 
 
+STREAM_ROWS = 64  # most rows of x one launch of the weight-streaming kernel takes
+
+
+def _streamed_float(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``x @ weight.T`` as unrounded float32 sums for any number of bfloat16 rows: the
+    weight-streaming kernel over groups of at most 64 rows (it re-reads ``weight`` once per
+    group)."""
+    if x.shape[0] <= STREAM_ROWS:
+        return gemm_skinny(x, weight, out_dtype=torch.float32)
+    out = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32, device=x.device)
+    for start in range(0, x.shape[0], STREAM_ROWS):
+        out[start: start + STREAM_ROWS] = gemm_skinny(x[start: start + STREAM_ROWS], weight,
+                                                      out_dtype=torch.float32)
+    return out
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """``x @ weight.T``.
 
-    bfloat16 by bfloat16: up to 16 rows go to the weight-streaming kernel, more rows to
-    the library matrix product (as the reference's ``nn.Linear`` does).  Every pairing
-    that involves float32 operands runs on the exact tiled kernel, which never uses a
-    reduced-precision matrix mode.
+    bfloat16 by bfloat16 with a bfloat16 result: up to 16 rows go to the weight-streaming
+    kernel, more rows to the library matrix product (as the reference's ``nn.Linear``
+    does); either way float32 sums are rounded once.  With a float32 result (the logits)
+    the sums come back unrounded whatever the number of rows, from the streaming kernel:
+    what a request's logits are rounded to does not depend on how many rows share its step.
+    Every pairing that involves float32 operands runs on the exact tiled kernel, which never
+    uses a reduced-precision matrix mode.
     """
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
@@ -503,30 +522,24 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.d
             raise KernelError("linear: operands must live on the GPU; there is no CPU path")
         if skinny_ok(x, weight):
             return gemm_skinny(x, weight, out_dtype=out_dtype)
+        if out_dtype == torch.float32 and _streaming_ok(x, weight, 1 << 30):
+            return _streamed_float(x, weight)
         y = torch.nn.functional.linear(x, weight)
         return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
     return gemm_tiled(x, weight, out_dtype=out_dtype)
 
 
 def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:
-    """A product whose result is about to be added to the residual stream: for few
-    rows it may come back as float32 partial sums ``[parts, M, N]``, which the fused
-    residual norm adds."""
+    """A product whose result is about to be added to the float32 residual stream.  For up
+    to 64 bfloat16 rows it comes back as unrounded float32 partial sums ``[parts, M, N]``,
+    which the fused residual norm adds; for more rows (prompt portions) it is the library's
+    product, rounded once to bfloat16."""
     if skinny_ok(x, weight):
         return gemm_skinny(x, weight, out_dtype=out_dtype, parts=k_parts(*weight.shape))
-    if _streaming_ok(x, weight, 64) and deep_or_small(*weight.shape):
+    if _streaming_ok(x, weight, STREAM_ROWS):
         n, k = weight.shape
         return gemm_skinny(x, weight, out_dtype=out_dtype, parts=8 if k >= 16384 else 4, row_tiles=4)
     return linear(x, weight, out_dtype=out_dtype)
-
-
-def deep_or_small(n: int, k: int) -> bool:
-    """Shapes at which, for 17 to 64 rows, the streaming kernel with K cut into parts beats
-    the library product: matrices much deeper than wide (a down projection; the library does
-    not cut K) and small ones (an out projection of a 4B or 8B model).  Measured at 64 rows:
-    2560x4096 14 against 19 us, 2560x9728 25 against 28, 4096x12288 32 against 37,
-    5120x25600 85 against 157; but 5120x8192 34 against 29, which stays with the library."""
-    return k >= 2 * n or n * k <= 24 * 1024 * 1024
 
 
 def linear_glu(x: torch.Tensor, gate_up: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:

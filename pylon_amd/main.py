@@ -143,22 +143,18 @@ def main(argv=None) -> None:
                          add_help=False)
     ben.add_argument("rest", nargs=argparse.REMAINDER)
 
-    sub.add_parser("selftest", help="generate a few tokens with a tiny random model and compare them with "
-                                    "the plain implementation (needs the repository's tests folder)")
+    sub.add_parser("selftest", help="run a tiny random model three ways that must agree (whole prompt against "
+                                    "token by token, bfloat16 against float32, the engine against a step loop)")
 
     args = parser.parse_args(argv)
     if args.command == "selftest":
-        root = Path(__file__).resolve().parent.parent
-        if str(root) not in sys.path:
-            sys.path.insert(0, str(root))
-        import torch
+        from .selftest import run as selftest
 
-        if not torch.cuda.is_available():
-            print("A GPU is required.", file=sys.stderr)
+        try:
+            selftest()
+        except RuntimeError as error:
+            print(error, file=sys.stderr)
             sys.exit(1)
-        import __graft_entry__
-
-        __graft_entry__.smoke()
         code = 0
     elif args.command == "generate":
         code = _generate(args)

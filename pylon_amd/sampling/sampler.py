@@ -84,7 +84,7 @@ class Sampler:
             for r, (s, index) in enumerate(rows):
                 params[0, r] = s.temperature
                 params[1, r] = s.top_p
-                params[2, r] = uniform(s.seed, index) if s.temperature > 0 else 0.0
+                params[2, r] = uniform(s.seed or 0, index) if s.temperature > 0 else 0.0
             dev = self._params_dev[k]
             dev.copy_(self._params_host[k], non_blocking=True)
             ops.sample(logits, dev[0, :n], dev[1, :n], dev[2, :n], out=out, chosen=chosen, place=place)

@@ -14,6 +14,7 @@ everything is float32.
 from __future__ import annotations
 
 import json
+import logging
 from pathlib import Path
 from typing import Dict, List, Tuple
 
@@ -21,6 +22,8 @@ import torch
 from safetensors import safe_open
 
 from ..config.registry import Architecture, WeightTarget
+
+logger = logging.getLogger("pylon")
 
 _FLOAT_STORED = {"F64", "F32", "F16", "BF16"}
 _INT_STORED = {"I64", "I32", "I16", "I8", "U8"}
@@ -64,9 +67,11 @@ def _param_dtype(model_dtype: torch.dtype, role: str, stored: List[str]) -> torc
     return torch.bfloat16
 
 
-def load_weights(model, arch: Architecture, config, folder) -> None:
+def load_weights(model, arch: Architecture, config, folder, *, strict: bool = False) -> List[str]:
     """Fill ``model``'s parameters from ``folder``; raise :class:`WeightsError` listing
-    every missing, unexpected and wrongly shaped tensor if the folder does not fit."""
+    every missing, wrongly shaped and unexpected tensor if a needed tensor is missing or
+    wrong (with ``strict``: also if only unexpected ones are found).  Returns the names of
+    the tensors that were skipped because the architecture does not know them."""
     folder = Path(folder)
     targets: Dict[str, WeightTarget] = arch.weight_targets(config)
     params = {path: (owner, name) for path, owner, name in model.named_params()}
@@ -101,8 +106,11 @@ def load_weights(model, arch: Architecture, config, folder) -> None:
                     continue
                 found[name] = (path, shape, stored)
     missing = [n for n, t in targets.items() if n not in present and not t.optional]
-    if missing or unexpected or wrong:
+    if missing or wrong or (strict and unexpected):
         raise WeightsError(missing, unexpected, wrong)
+    if unexpected:
+        logger.warning("weights_skipped folder=%s count=%d names=%s", folder, len(unexpected),
+                       ", ".join(sorted(unexpected)[:8]) + (" ..." if len(unexpected) > 8 else ""))
 
     # Decide each parameter's element type from what is stored for it, then copy.
     stored_by_param: Dict[str, List[str]] = {}
@@ -132,3 +140,4 @@ def load_weights(model, arch: Architecture, config, folder) -> None:
                     dest = dest[target.row_start: target.row_start + tensor.shape[0]]
                 dest.copy_(tensor.to(dest.dtype))
                 filled[target.param] = filled.get(target.param, 0) + 1
+    return sorted(unexpected)

@@ -19,11 +19,44 @@ from safetensors.torch import save_file
 from ..config.registry import resolve
 
 
-def _generator(seed: int, name: str) -> torch.Generator:
+def _generator(seed: int, name: str, device="cpu") -> torch.Generator:
     digest = hashlib.sha256(f"{seed}:{name}".encode()).digest()
-    gen = torch.Generator(device="cpu")
+    gen = torch.Generator(device=device)
     gen.manual_seed(int.from_bytes(digest[:8], "little") & ((1 << 63) - 1))
     return gen
+
+
+_SLAB = 1 << 26  # elements drawn at a time, so that no float32 copy of a large matrix is needed
+
+
+def draw_tensor(seed: int, name: str, target, sigma: float, norm_jitter: float, *, out: torch.Tensor) -> None:
+    """The one rule of the random-weights mode: fill ``out`` (of the target's shape, on any
+    device, of any float type) with tensor ``name`` of seed ``seed``.  ``normal``:
+    N(0, sigma^2); ``ones`` / ``ones_jitter``: 1, or 1 + norm_jitter * N(0, 1).  The numbers
+    come from a generator on ``out``'s device keyed by (seed, name): a folder written on the
+    CPU and a model filled on the GPU follow the same rule, but not the same numbers."""
+    if tuple(out.shape) != tuple(target.shape):
+        raise ValueError(f"{name}: expected a tensor of shape {tuple(target.shape)}, got {tuple(out.shape)}")
+    if target.init in ("ones", "ones_jitter") and not (target.init == "ones_jitter" and norm_jitter):
+        out.fill_(1.0)
+        return
+    if target.init not in ("normal", "ones_jitter"):
+        raise ValueError(f"unknown init rule {target.init!r} for {name}")
+    gen = _generator(seed, name, out.device)
+    scale, shift = (sigma, 0.0) if target.init == "normal" else (norm_jitter, 1.0)
+    if out.is_contiguous():
+        flat = out.view(-1)
+        for start in range(0, flat.numel(), _SLAB):
+            part = flat[start: start + _SLAB]
+            part.copy_(torch.randn(part.numel(), generator=gen, dtype=torch.float32, device=out.device)
+                       * scale + shift)
+    else:
+        out.copy_(torch.randn(tuple(out.shape), generator=gen, dtype=torch.float32, device=out.device)
+                  * scale + shift)
+
+
+def _sigma(cfg, std: Optional[float]) -> float:
+    return float(std if std is not None else getattr(cfg, "initializer_range", 0.02))
 
 
 def write_random_model(folder, config: Mapping, seed: int, *, dtype: str = "bfloat16",
@@ -40,23 +73,41 @@ def write_random_model(folder, config: Mapping, seed: int, *, dtype: str = "bflo
     store = torch.bfloat16 if dtype == "bfloat16" else torch.float32
     arch = resolve(config)
     cfg = arch.parse_config(config)
-    sigma = float(std if std is not None else getattr(cfg, "initializer_range", 0.02))
+    sigma = _sigma(cfg, std)
     tensors = {}
     for name, target in arch.weight_targets(cfg).items():
         if target.init == "skip":
             continue
-        gen = _generator(seed, name)
-        if target.init == "normal":
-            value = torch.randn(target.shape, generator=gen, dtype=torch.float32) * sigma
-        elif target.init in ("ones", "ones_jitter"):
-            value = torch.ones(target.shape, dtype=torch.float32)
-            if target.init == "ones_jitter" and norm_jitter:
-                value += norm_jitter * torch.randn(target.shape, generator=gen, dtype=torch.float32)
-        else:
-            raise ValueError(f"unknown init rule {target.init!r} for {name}")
+        value = torch.empty(target.shape, dtype=torch.float32)
+        draw_tensor(seed, name, target, sigma, norm_jitter, out=value)
         tensors[name] = value.to(store).contiguous()
     folder = Path(folder)
     folder.mkdir(parents=True, exist_ok=True)
     (folder / "config.json").write_text(json.dumps(arch.config_to_json(cfg), indent=2) + "\n")
     save_file(tensors, str(folder / "model.safetensors"))
     return folder
+
+
+def fill_random_model(model, arch, cfg, seed: int, *, std: Optional[float] = None,
+                      norm_jitter: float = 0.0) -> None:
+    """The same mode without the folder: fill ``model``'s parameters in place, on their
+    device, tensor by tensor through the architecture's table of checkpoint names (so fused
+    matrices get their parts in their row ranges, as a load would put them).  For models too
+    large to be worth writing to disk; every parameter must be covered."""
+    params = {path: (owner, name) for path, owner, name in model.named_params()}
+    sigma = _sigma(cfg, std)
+    covered = {path: 0 for path in params}
+    for name, target in arch.weight_targets(cfg).items():
+        if target.init == "skip":
+            continue
+        if target.param not in params:
+            raise ValueError(f"{name}: the model has no parameter {target.param}")
+        owner, pname = params[target.param]
+        dest = owner.params[pname]
+        if dest.dim() >= 1 and len(target.shape) >= 1 and tuple(dest.shape) != tuple(target.shape):
+            dest = dest[target.row_start: target.row_start + target.shape[0]]
+        draw_tensor(seed, name, target, sigma, norm_jitter, out=dest)
+        covered[target.param] += dest.numel()
+    short = [path for path, (owner, pname) in params.items() if covered[path] != owner.params[pname].numel()]
+    if short:
+        raise ValueError("the architecture's table of tensors does not cover: " + ", ".join(sorted(short)))

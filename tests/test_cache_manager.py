@@ -249,3 +249,61 @@ def test_mixed_step_metadata_and_refusals():
         _ctx(m, [StepEntry(b, list(range(40)), [])])
     assert m.free_pages == free
     m.check()
+
+
+def test_a_failure_after_the_pages_were_taken_gives_them_back():
+    # the metadata upload fails (as a device error would): the step's pages return to the
+    # pool, no append stays pending, and the next step runs
+    m = make(page_size=4, num_pages=8)
+    a = m.open("a")
+    feed(m, a, 3)
+    free = m.free_pages
+
+    class FailingArena(MetadataArena):
+        def upload(self, index, size, into=None):
+            raise RuntimeError("device lost")
+
+    with pytest.raises(RuntimeError, match="device lost"):
+        build_step([StepEntry(a, [1, 2, 3], [2])], m, FailingArena("cpu", capacity=256), vocab_size=100)
+    assert m.free_pages == free and a._pending is None
+    m.check()
+    with pytest.raises(ValueError, match="block table holds"):
+        _ctx(m, [StepEntry(a, [1, 2, 3], [2])], width=1)
+    assert m.free_pages == free and a._pending is None
+    ctx = _ctx(m, [StepEntry(a, [1, 2, 3], [2])])
+    assert ctx.positions.tolist() == [3, 4, 5]
+    m.commit([(a, 3)])
+    m.check()
+
+
+def test_a_replay_that_raises_leaves_the_cache_as_it_was():
+    from pylon_amd.engine.graphs import DecodeGraphs
+
+    m = make(page_size=4, num_pages=8)
+    a = m.open("a")
+    feed(m, a, 4)  # the next token opens a second page
+    free = m.free_pages
+
+    class Spec:
+        vocab_size = 100
+
+    class FakeModel:
+        spec = Spec()
+        device = torch.device("cpu")
+
+    class BrokenGraph:
+        def replay(self):
+            raise RuntimeError("replay failed")
+
+    graphs = DecodeGraphs.__new__(DecodeGraphs)
+    graphs.model, graphs.manager, graphs.arena = FakeModel(), m, MetadataArena("cpu", capacity=256)
+    graphs.chosen, graphs.width, graphs.max_batch = None, 4, 4
+    graphs.failed, graphs.replays, graphs.last_logit_slots = set(), 0, None
+    block = torch.empty(256, dtype=torch.int32)
+    graphs.captured = {(1, 1024): (BrokenGraph(), block, None, None)}
+    with pytest.raises(RuntimeError, match="replay failed"):
+        graphs.run([StepEntry(a, [7], [0])])
+    assert m.free_pages == free and a._pending is None and a.length == 4
+    m.check()
+    ctx = _ctx(m, [StepEntry(a, [7], [0])])
+    assert ctx.positions.tolist() == [4]

@@ -136,8 +136,16 @@ def test_serving_config_defaults_and_checks(monkeypatch):
     assert env.prefill_chunk_size == 512 and env.cuda_graphs is True and env.admit_skip == 2
     assert get_config(prefill_chunk_size=64).prefill_chunk_size == 64
     monkeypatch.setenv("PYLON_CUDA_GRAPHS", "yes")
-    with pytest.raises(ValueError, match="must be true, false, 1, or 0"):
+    with pytest.raises(ValueError, match="PYLON_CUDA_GRAPHS = 'yes' cannot be read: expected true, false, 1 or 0"):
         get_config()
+    monkeypatch.setenv("PYLON_CUDA_GRAPHS", "0")
+    monkeypatch.setenv("PYLON_NUM_PAGES", "")
+    monkeypatch.setenv("PYLON_MAX_BATCH_SIZE", "0")
+    with pytest.raises(ValueError, match="max_batch_size = 0 is not allowed: it must be a whole number of at least 1"):
+        get_config()
+    assert get_config(max_batch_size=3).num_pages is None  # an argument wins over the variable
+    with pytest.raises(TypeError, match="unknown option"):
+        get_config(no_such_option=1)
 
 
 def test_weights_must_fit_under_the_utilisation_limit():

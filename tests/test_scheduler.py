@@ -514,3 +514,40 @@ def test_run_ahead_cancellation_and_failure_with_a_step_in_flight():
     fc = enqueue(engine, "c", [1], 2)
     engine.run_until_idle()
     assert fc.result(timeout=0).output_ids == [7, 7]
+
+
+def test_a_request_without_a_seed_gets_one_of_its_own_and_a_given_seed_is_kept():
+    engine, runner, clock = make_engine()
+    seen = {}
+
+    class Recording(ScriptedSampler):
+        def sample(self, logits, rows):
+            for rid, (sampling, _index) in zip(logits, rows):
+                seen.setdefault(rid, set()).add(sampling.seed)
+            return super().sample(logits, rows)
+
+    engine.sampler = Recording()
+    hot = Sampling(max_new_tokens=3, temperature=0.8)
+    futures = [engine.enqueue([1, 2, 3], None, hot, "a"), engine.enqueue([1, 2, 3], None, hot, "b"),
+               engine.enqueue([1, 2, 3], None, Sampling(max_new_tokens=3, temperature=0.8, seed=5), "c"),
+               engine.enqueue([1, 2, 3], None, Sampling(max_new_tokens=3, temperature=0.8, seed=5), "d")]
+    engine.run_until_idle()
+    assert all(f.done() for f in futures)
+    (a,), (b,) = seen["a"], seen["b"]  # one seed for the whole of a request
+    assert a != b and a is not None and b is not None  # two unseeded equal prompts differ
+    assert seen["c"] == {5} and seen["d"] == {5}  # a given seed is kept, so it repeats
+    with pytest.raises(ValueError):
+        Sampling(seed=-1)
+
+
+def test_results_carry_the_reference_timing_fields():
+    # /root/reference/src/pylon/engine.py:59-74, 598-618: first_token_at on the engine's clock,
+    # token_intervals between emitted tokens (one fewer than the tokens)
+    engine, runner, clock = make_engine()
+    future = enqueue(engine, "a", [1, 2, 3], 4)
+    while engine.tick():
+        clock.now += 0.25
+    result = future.result()
+    assert len(result.output_ids) == 4 and len(result.token_intervals) == 3
+    assert result.first_token_at == pytest.approx(1000.0 + result.first_token_seconds)
+    assert all(abs(dt - 0.25) < 1e-9 for dt in result.token_intervals)

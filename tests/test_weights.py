@@ -95,6 +95,25 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     assert "model.norm.weight" in text and "rotary_emb" in text
 
 
+def test_a_tensor_the_architecture_does_not_know_is_skipped(tmp_path, caplog):
+    # /root/reference/src/pylon/model/weights.py:22-25 passes over names it has no target for
+    folder = make_model_folder(tmp_path, "A", dtype="float32")
+    raw = load_file(str(folder / "model.safetensors"))
+    raw["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    save_file(raw, str(folder / "model.safetensors"))
+    arch, cfg = load_model_config(folder)
+    model = Model(arch.model_spec(cfg), dtype=torch.float32, device="cpu")
+    with caplog.at_level("WARNING", logger="pylon"):
+        skipped = load_weights(model, arch, cfg, folder)
+    assert skipped == ["model.layers.0.self_attn.rotary_emb.inv_freq"]
+    assert "rotary_emb.inv_freq" in caplog.text
+    assert torch.equal(model.params["embed"], raw["model.embed_tokens.weight"])
+    with pytest.raises(WeightsError) as info:  # on request it is an error of its own
+        load_weights(Model(arch.model_spec(cfg), dtype=torch.float32, device="cpu"), arch, cfg, folder,
+                     strict=True)
+    assert info.value.unexpected == skipped and not info.value.missing
+
+
 def test_tied_head_is_optional_and_untied_head_is_required(tmp_path):
     folder = make_model_folder(tmp_path, "A", dtype="float32")
     raw = load_file(str(folder / "model.safetensors"))
@@ -126,3 +145,18 @@ def test_sharded_folder_and_missing_file(tmp_path):
     (folder / "model-00002-of-00002.safetensors").unlink()
     with pytest.raises(FileNotFoundError):
         _load(folder, torch.float32)
+
+
+def test_filling_a_model_in_place_follows_the_folder_rule(tmp_path):
+    # on the CPU the two ways of the random-weights mode give the same numbers
+    from pylon_amd.weights import fill_random_model
+
+    folder = write_random_model(tmp_path / "m", TINY_B, 5, dtype="float32", norm_jitter=0.2)
+    loaded = _load(folder, torch.float32)
+    arch, cfg = load_model_config(folder)
+    filled = Model(arch.model_spec(cfg), dtype=torch.float32, device="cpu")
+    for _, owner, name in filled.named_params():
+        owner.params[name].fill_(float("nan"))
+    fill_random_model(filled, arch, cfg, 5, norm_jitter=0.2)
+    for (path, a_owner, a_name), (_, b_owner, b_name) in zip(loaded.named_params(), filled.named_params()):
+        assert torch.equal(a_owner.params[a_name], b_owner.params[b_name]), path
