@@ -245,7 +245,9 @@ def engine_run(runner, cfg, batch: int, seed: int, prompt_len: int = PROMPT_LEN,
     engine = Engine(PylonConfig(max_batch_size=batch, max_queue_size=batch, page_size=PAGE_SIZE), runner=runner)
     sampling = Sampling(max_new_tokens=new_tokens, temperature=0.0)
     if runner.graphs is not None:  # as a server does at start-up
-        runner.capture_graphs(range(1, batch + 1))
+        longest = prompt_len + new_tokens
+        runner.capture_graphs(range(1, batch + 1),
+                              bounds=[b for b in runner.graphs.bounds() if b < 2 * longest])
     torch.cuda.synchronize()
     started = time.perf_counter()
     results = engine.generate(prompts, sampling)

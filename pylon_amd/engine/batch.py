@@ -106,6 +106,7 @@ class StepContext:
     fixed_shapes: bool = False  # launches must not depend on lengths (graph capture)
     logit_slots: Optional[torch.Tensor] = None  # int32 [n]: state slot of each wanted row's request
     chosen: Optional[torch.Tensor] = None  # int32 [slots]: last sampled token per state slot
+    logits_out: Optional[torch.Tensor] = None  # float32 [>= n_logits, vocab]: where the logits go, if given
     _tiles: Dict[Tuple[int, int], torch.Tensor] = field(default_factory=dict)
 
     def cache(self, cache_id: int) -> CacheView:

@@ -41,6 +41,9 @@ class DecodeGraphs:
         self.max_batch = max_batch
         self.width = max_pages_per_request
         self.pool = torch.cuda.graph_pool_handle()
+        # Every graph leaves its logits in the first rows of this one buffer: with a buffer per
+        # graph, the graphs of a large vocabulary would hold gigabytes between them.
+        self.logits = torch.empty((max_batch, model.spec.vocab_size), dtype=torch.float32, device=model.device)
         self.captured: Dict[Tuple[int, int], tuple] = {}
         self.failed = set()
         self.replays = 0
@@ -96,6 +99,7 @@ class DecodeGraphs:
             ctx = build_step(entries, manager, arena, vocab_size=model.spec.vocab_size,
                              width=self.width, device_block=block, fixed_shapes=True,
                              chosen=self.chosen, len_bound=bound)
+            ctx.logits_out = self.logits
             # No garbage collection while the stream is capturing: a finalizer that frees a
             # device object (an event, another graph) is not allowed there and aborts.
             gc.collect()

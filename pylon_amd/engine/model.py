@@ -70,4 +70,5 @@ class Model(Part):
         if ctx.n_logits == 0:
             return None
         h = self.final_norm.add_forward(resid, delta, row_idx=ctx.logit_idx)
-        return ops.linear(h, self.head_weight, out_dtype=torch.float32)
+        out = None if ctx.logits_out is None else ctx.logits_out[: ctx.n_logits]
+        return ops.linear(h, self.head_weight, out_dtype=torch.float32, out=out)

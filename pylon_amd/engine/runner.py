@@ -50,6 +50,22 @@ def check_weights_fit(needed: int, free: int, total: int, config, what) -> None:
             f"{available:,} bytes are available under the GPU utilization limit.")
 
 
+def pool_pages(free: int, total: int, bytes_per_token: int, config, max_positions: Optional[int]) -> int:
+    """Pages of the cache pool from the device's memory once the weights are resident
+    (/root/reference/src/pylon/kv/budget.py:70-113): the utilisation limit times the total,
+    minus what is occupied, minus a headroom ``free - free / (1 + kv_cache_headroom_ratio)``
+    that stays free for activations and graphs; no more than ``max_batch_size`` requests of
+    the model's longest length could ever hold."""
+    headroom = free - int(free / (1 + config.kv_cache_headroom_ratio))
+    budget = math.floor(total * config.max_gpu_utilization) - (total - free) - headroom
+    pages = budget // max(1, config.page_size * bytes_per_token)
+    if max_positions:
+        pages = min(pages, -(-max_positions // config.page_size) * config.max_batch_size)
+    if pages < 1:
+        raise RuntimeError("Not enough GPU memory remains for the KV cache and activations.")
+    return int(pages)
+
+
 class Runner:
     def __init__(self, model: Model, *, page_size: int, num_pages: int, max_requests: int) -> None:
         if model.device.type != "cuda":
@@ -96,21 +112,18 @@ class Runner:
         model = Model(spec, dtype=resolve_dtype(config.dtype), device=device)
         load_weights(model, arch, model_config, Path(config.model_path))
         num_pages = config.num_pages
+        sizing = None
         if num_pages is None:
             from ..cache.manager import bytes_per_token
 
             per_token = bytes_per_token(model.cache_requirements(), model.dtype)
             free, total = torch.cuda.mem_get_info(model.device)
-            budget = int(total * config.max_gpu_utilization) - (total - free)
-            budget = int(budget * (1.0 - config.kv_cache_headroom_ratio))
-            num_pages = budget // max(1, config.page_size * per_token)
-            ceiling = -(-model.spec.max_positions // config.page_size) * config.max_batch_size
-            num_pages = min(num_pages, ceiling)
-            if num_pages < 1:
-                raise ValueError("The KV budget must hold at least one attention page.")
+            num_pages = pool_pages(free, total, per_token, config, model.spec.max_positions)
+            sizing = {"free": free, "total": total, "bytes_per_token": per_token, "num_pages": num_pages}
         runner = cls(model, page_size=config.page_size, num_pages=int(num_pages),
                      max_requests=config.max_batch_size)
         runner.config = model_config
+        runner.pool_sizing = sizing  # what the pool was sized from (None: num_pages was given)
         if config.cuda_graphs:
             runner.enable_graphs(config.max_batch_size)
             runner.capture_graphs()
@@ -133,7 +146,10 @@ class Runner:
         """Capture decode graphs now instead of at their first use, as the reference does at
         start-up (/root/reference/src/pylon/decode/warmup.py:140-167): for these batch sizes
         (default: every size the graphs serve) and these bounds on the requests' lengths
-        (default: every bound, see :meth:`DecodeGraphs.bounds`).  Throw-away requests of one
+        (default: the smallest, which serves requests of up to 1,024 tokens; the graphs of
+        longer requests, see :meth:`DecodeGraphs.bounds`, are captured when such a request
+        first decodes: a model of 262,144 positions has nine bounds, and start-up would
+        capture nine graphs per batch size).  Throw-away requests of one
         token each take one decode step per graph and are closed again.  Sizes for which the
         pool has no free pages or slots are left to their first use.  Returns the batch sizes
         that have a graph."""
@@ -142,7 +158,7 @@ class Runner:
         from ..cache import OutOfPages
 
         sizes = sorted(set(batch_sizes or range(1, self.graphs.max_batch + 1)))
-        bounds = sorted(set(bounds or self.graphs.bounds()))
+        bounds = sorted(set(bounds or self.graphs.bounds()[:1]))
         most = min(max(sizes), self.manager.free_pages, self.manager.slots.free_slots, self.graphs.max_batch)
         seqs = [self.open(("graph-warm-up", i)) for i in range(most)]
         limit = self.model.spec.max_positions

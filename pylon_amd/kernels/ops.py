@@ -448,7 +448,8 @@ def skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
 
 
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype = torch.bfloat16,
-                parts: int = 1, glu: bool = False, row_tiles: int = 0) -> torch.Tensor:
+                parts: int = 1, glu: bool = False, row_tiles: int = 0,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ weight.T`` for at most 64 rows of bfloat16 ``x``, streaming ``weight`` once.
 
     ``parts > 1`` cuts K into that many ranges and returns float32 partial results
@@ -469,10 +470,12 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype
         raise KernelError("gemm_skinny takes bfloat16 operands")
     if not (x.is_cuda and weight.is_cuda) or x.stride(1) != 1 or weight.stride(1) != 1:
         raise KernelError("gemm_skinny: operands must be on the GPU with contiguous rows")
-    if parts > 1:
-        out = torch.empty((parts, m, n), dtype=torch.float32, device=x.device)
-    else:
-        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    shape = (parts, m, n) if parts > 1 else (m, n)
+    if out is None:
+        out = torch.empty(shape, dtype=torch.float32 if parts > 1 else out_dtype, device=x.device)
+    elif tuple(out.shape) != shape or out.dtype != (torch.float32 if parts > 1 else out_dtype) \
+            or not out.is_cuda or not out.is_contiguous():
+        raise KernelError(f"gemm_skinny: out must be contiguous, on the GPU and of shape {shape}")
     _lib.call("pylon_gemm_skinny", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), weight.data_ptr(),
               m, n, k, x.stride(0), weight.stride(0), n, parts, m * n, 1 if glu else 0, int(row_tiles), _stream())
     return out
@@ -492,21 +495,23 @@ def k_parts(n: int, k: int) -> int:
 STREAM_ROWS = 64  # most rows of x one launch of the weight-streaming kernel takes
 
 
-def _streamed_float(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+def _streamed_float(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ weight.T`` as unrounded float32 sums for any number of bfloat16 rows: the
     weight-streaming kernel over groups of at most 64 rows (it re-reads ``weight`` once per
     group)."""
     if x.shape[0] <= STREAM_ROWS:
-        return gemm_skinny(x, weight, out_dtype=torch.float32)
-    out = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32, device=x.device)
+        return gemm_skinny(x, weight, out_dtype=torch.float32, out=out)
+    if out is None:
+        out = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32, device=x.device)
     for start in range(0, x.shape[0], STREAM_ROWS):
-        out[start: start + STREAM_ROWS] = gemm_skinny(x[start: start + STREAM_ROWS], weight,
-                                                      out_dtype=torch.float32)
+        gemm_skinny(x[start: start + STREAM_ROWS], weight, out_dtype=torch.float32,
+                    out=out[start: start + STREAM_ROWS])
     return out
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """``x @ weight.T``.
+def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.dtype] = None,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x @ weight.T`` (into ``out`` if given: contiguous, of the result's shape and type).
 
     bfloat16 by bfloat16 with a bfloat16 result: up to 16 rows go to the weight-streaming
     kernel, more rows to the library matrix product (as the reference's ``nn.Linear``
@@ -521,12 +526,13 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.d
         if not x.is_cuda:
             raise KernelError("linear: operands must live on the GPU; there is no CPU path")
         if skinny_ok(x, weight):
-            return gemm_skinny(x, weight, out_dtype=out_dtype)
+            return gemm_skinny(x, weight, out_dtype=out_dtype, out=out)
         if out_dtype == torch.float32 and _streaming_ok(x, weight, 1 << 30):
-            return _streamed_float(x, weight)
+            return _streamed_float(x, weight, out)
         y = torch.nn.functional.linear(x, weight)
-        return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
-    return gemm_tiled(x, weight, out_dtype=out_dtype)
+        y = y if out_dtype == torch.bfloat16 else y.to(out_dtype)
+        return y if out is None else out.copy_(y)
+    return gemm_tiled(x, weight, out_dtype=out_dtype, out=out)
 
 
 def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:

@@ -89,3 +89,16 @@ def read_folder(folder: Path):
 
 def random_tokens(vocab: int, count: int, seed: int):
     return np.random.default_rng(seed).integers(0, vocab, count).tolist()
+
+
+def rows_within(got, ref, bound: float):
+    """Every row of ``got`` is within ``bound`` times that row's own largest |reference logit|
+    of ``ref`` (a bad row cannot hide under another row's large logit).  Returns
+    (ok, index of the worst row, its error as a fraction of its scale)."""
+    got, ref = np.asarray(got), np.asarray(ref)
+    if got.ndim == 1:
+        got, ref = got[None], ref[None]
+    assert got.shape == ref.shape, (got.shape, ref.shape)
+    frac = np.abs(got - ref).max(axis=1) / np.abs(ref).max(axis=1)
+    worst = int(frac.argmax())
+    return bool(frac[worst] <= bound), worst, float(frac[worst])

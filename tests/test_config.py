@@ -183,3 +183,22 @@ def test_stop_ids_come_from_generation_config_before_config(tmp_path):
     assert read_stop_token_ids(tmp_path) == (7,)
     (tmp_path / "config.json").write_text(json.dumps(TINY_A))
     assert read_stop_token_ids(tmp_path) == ()
+
+
+def test_pool_pages_follow_the_reference_budget():
+    """/root/reference/src/pylon/kv/budget.py:70-113 with its own numbers: utilisation limit
+    times total, minus what is occupied, minus free - free/(1 + ratio)."""
+    from pylon_amd.config import PylonConfig
+    from pylon_amd.engine.runner import pool_pages
+
+    config = PylonConfig(page_size=16, max_batch_size=4, max_gpu_utilization=0.9, kv_cache_headroom_ratio=0.25)
+    total, free = 1000_000, 600_000
+    headroom = free - int(free / 1.25)  # 120,000
+    budget = 900_000 - 400_000 - headroom  # 380,000
+    assert pool_pages(free, total, 100, config, None) == budget // 1600
+    assert pool_pages(free, total, 100, config, 64) == 4 * 4  # four requests of the longest length
+    assert pool_pages(free, total, 100, config, 70) == 4 * 5
+    import pytest
+
+    with pytest.raises(RuntimeError, match="Not enough GPU memory"):
+        pool_pages(free, total, 100_000, config, None)

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests.helpers import make_model_folder, random_tokens, read_folder
+from tests.helpers import make_model_folder, random_tokens, read_folder, rows_within
 from tests.plain import qwen3 as plain
 
 pytestmark = pytest.mark.gpu
@@ -64,10 +64,8 @@ def test_benchmark_layer_sizes_match_the_plain_model(real, dtype, bound):
     assert runner.graphs.replays >= 20 and set(runner.graphs.captured_sizes()) == {1, 2, 3}
     for i, ref in enumerate(want):
         g = np.concatenate(got[i])
-        scale = np.abs(ref).max()
         assert len(g) == len(ref)
-        err = np.abs(g - ref).max(axis=1)
-        assert err.max() <= bound * scale, (dtype, i, int(err.argmax()), float(err.max()), float(scale))
+        assert rows_within(g, ref, bound)[0], (dtype, i, rows_within(g, ref, bound))
 
 
 @pytest.mark.parametrize("dtype,bound", [("float32", 2e-5), ("bfloat16", 3e-2)])
@@ -92,8 +90,7 @@ def test_twenty_requests_decode_side_by_side(real, dtype, bound):
     assert runner.graphs.captured_sizes() == (20,) and runner.graphs.replays == decoded
     for i, ref in enumerate(want):
         got = np.stack([rows[t][i] for t in range(decoded)])
-        scale = np.abs(ref).max()
-        assert np.abs(got - ref[-decoded:]).max() <= bound * scale, (dtype, i)
+        assert rows_within(got, ref[-decoded:], bound)[0], (dtype, i, rows_within(got, ref[-decoded:], bound))
 
 
 WIDE = dict(REAL, num_hidden_layers=1, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8,
@@ -125,4 +122,4 @@ def test_a_layer_of_the_widest_shape(tmp_path):
         n = len(requests[i]) - decoded
         got = np.concatenate([first[at: at + n], np.stack([rows[t][i] for t in range(decoded)])])
         at += n
-        assert np.abs(got - ref).max() <= 3e-2 * np.abs(ref).max(), i
+        assert rows_within(got, ref, 3e-2)[0], (i, rows_within(got, ref, 3e-2))
