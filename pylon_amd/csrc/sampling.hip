@@ -21,6 +21,9 @@
 //   4. the cumulative mass of kept tokens in index order, narrowed from the row to a
 //      sixteenth of it twice and then scanned.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 typedef unsigned long long u64;
 
@@ -163,6 +166,50 @@ extern "C" int pylon_argmax(int* out, const float* logits, int rows, int vocab, 
   hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(PYLON_WAVE), 0, stream, out,
                      static_cast<const ArgBest*>(scratch), chunks, chosen, place);
   PYLON_LAUNCHED("argmax");
+}
+
+// ---- argmax without a scratch argument -----------------------------------------------------
+// The first launch's partial results in an array of the library's own.  In host code the
+// array's name is only a stand-in for the symbol; the address on a device comes from
+// hipGetSymbolAddress, once per device, and only that address is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[PYLON_ARGMAX_STATIC_MAX_ROWS * ARGMAX_MAX_CHUNKS *
+                                                        sizeof(ArgBest)];
+#define STATIC_MAX_DEVICES 64
+static void* static_scratch_ptr[STATIC_MAX_DEVICES];  // by device ordinal; null: not resolved yet
+static std::mutex static_scratch_lock;
+
+static int static_scratch(void** ptr) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) PYLON_REFUSE("argmax_static: no current device: %s", hipGetErrorString(e));
+  PYLON_REQUIRE(dev >= 0 && dev < STATIC_MAX_DEVICES, "argmax_static: device ordinal %d is beyond %d", dev,
+                STATIC_MAX_DEVICES);
+  std::lock_guard<std::mutex> guard(static_scratch_lock);
+  if (static_scratch_ptr[dev] == nullptr) {
+    void* found = nullptr;
+    e = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || found == nullptr)
+      PYLON_REFUSE("argmax_static: the scratch array has no address on device %d: %s", dev, hipGetErrorString(e));
+    static_scratch_ptr[dev] = found;
+  }
+  *ptr = static_scratch_ptr[dev];
+  return 0;
+}
+
+extern "C" int pylon_argmax_static_init(void) {
+  void* ptr = nullptr;
+  return static_scratch(&ptr);
+}
+
+extern "C" int pylon_argmax_static(int* out, const float* logits, int rows, int vocab, long long row_stride,
+                                   int* chosen, const int* place, hipStream_t stream) {
+  PYLON_REQUIRE(rows <= PYLON_ARGMAX_STATIC_MAX_ROWS,
+                "argmax_static: takes at most %d rows (the size of its fixed scratch array), got %d",
+                PYLON_ARGMAX_STATIC_MAX_ROWS, rows);
+  void* ptr = nullptr;
+  if (static_scratch(&ptr)) return 1;
+  return pylon_argmax(out, logits, rows, vocab, row_stride, chosen, place, ptr,
+                      static_cast<long long>(sizeof(scratch)), stream);
 }
 
 // ---- sample ------------------------------------------------------------------------------
