@@ -105,8 +105,10 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
   const int c_end = c_begin + per_cut < pos + 1 ? c_begin + per_cut : pos + 1;
   const bool holds_last = pos >= c_begin && pos < c_begin + per_cut;  // true for exactly one cut
   const int n_keys = c_end > c_begin ? c_end - c_begin : 0;
+  // A wave's range is a whole number of the batches it loads at once: with few keys, fewer
+  // waves take part, rather than all of them loading a mostly empty batch each.
   int per_wave = (n_keys + n_waves - 1) / n_waves;
-  per_wave = (per_wave + AD_TILE - 1) / AD_TILE * AD_TILE;
+  per_wave = (per_wave + SUPER - 1) / SUPER * SUPER;
   const int k_begin = c_begin + wave * per_wave;
   int k_end = k_begin + per_wave;
   if (k_end > c_end) k_end = c_end;

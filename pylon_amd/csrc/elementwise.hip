@@ -260,8 +260,8 @@ extern "C" int pylon_residual_add(float* resid, const void* delta, int delta_dty
 
 // ---- gated activation -----------------------------------------------------------------
 // out[t, i] = silu(gu[t, i]) * gu[t, inter + i]; silu(z) = z / (1 + exp(-z)).
-template <typename T>
-__global__ void silu_gate_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter, size_t total) {
+template <typename TI, typename TO>
+__global__ void silu_gate_kernel(TO* __restrict__ out, const TI* __restrict__ gu, int inter, size_t total) {
   size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
   for (; i < total; i += step) {
@@ -270,7 +270,7 @@ __global__ void silu_gate_kernel(T* __restrict__ out, const T* __restrict__ gu, 
     const float g = to_float(gu[t * 2 * inter + c]);
     const float u = to_float(gu[t * 2 * inter + inter + c]);
     const float s = g / (1.0f + expf(-g));
-    out[i] = from_float<T>(s * u);
+    out[i] = from_float<TO>(s * u);
   }
 }
 
@@ -298,14 +298,16 @@ __global__ void silu_gate_bf16x8_kernel(uint4* __restrict__ out, const uint4* __
   }
 }
 
-extern "C" int pylon_silu_gate(void* out, const void* gate_up, int dtype, int tokens, int inter,
+// gate_up: [tokens, 2 * inter] of in_dtype; out: [tokens, inter] of out_dtype (float sums of a
+// product may come in as float and leave as bfloat16: one rounding, after the activation).
+extern "C" int pylon_silu_gate(void* out, int out_dtype, const void* gate_up, int in_dtype, int tokens, int inter,
                                hipStream_t stream) {
-  PYLON_REQUIRE(pylon_valid_dtype(dtype), "silu_gate: unknown dtype");
+  PYLON_REQUIRE(pylon_valid_dtype(in_dtype) && pylon_valid_dtype(out_dtype), "silu_gate: unknown dtype");
   PYLON_REQUIRE(tokens >= 0 && inter > 0, "silu_gate: bad sizes tokens=%d inter=%d", tokens, inter);
   const size_t total = static_cast<size_t>(tokens) * inter;
   if (total == 0) return 0;
-  if (dtype == PYLON_BF16 && inter % 8 == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
-      (reinterpret_cast<uintptr_t>(gate_up) & 15) == 0) {
+  if (in_dtype == PYLON_BF16 && out_dtype == PYLON_BF16 && inter % 8 == 0 &&
+      (reinterpret_cast<uintptr_t>(out) & 15) == 0 && (reinterpret_cast<uintptr_t>(gate_up) & 15) == 0) {
     const size_t chunks_total = total / 8;
     size_t nblocks = (chunks_total + 255) / 256;
     if (nblocks > 65535u * 16u) nblocks = 65535u * 16u;
@@ -316,11 +318,12 @@ extern "C" int pylon_silu_gate(void* out, const void* gate_up, int dtype, int to
   size_t blocks = (total + 255) / 256;
   if (blocks > 65535u * 16u) blocks = 65535u * 16u;
   dim3 grid((unsigned)blocks), block(256);
-  if (dtype == PYLON_F32)
-    hipLaunchKernelGGL(silu_gate_kernel<float>, grid, block, 0, stream, (float*)out, (const float*)gate_up,
-                       inter, total);
-  else
-    hipLaunchKernelGGL(silu_gate_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)out,
-                       (const bf16_t*)gate_up, inter, total);
+#define GO(TI, TO) \
+  hipLaunchKernelGGL((silu_gate_kernel<TI, TO>), grid, block, 0, stream, (TO*)out, (const TI*)gate_up, inter, total)
+  if (in_dtype == PYLON_F32 && out_dtype == PYLON_F32) GO(float, float);
+  else if (in_dtype == PYLON_F32) GO(float, bf16_t);
+  else if (out_dtype == PYLON_F32) GO(bf16_t, float);
+  else GO(bf16_t, bf16_t);
+#undef GO
   PYLON_LAUNCHED("silu_gate");
 }

@@ -29,7 +29,7 @@ _SIGNATURES = {
     "pylon_rmsnorm": [P, I, P, I, P, P, I, I, F, P],
     "pylon_add_rmsnorm": [P, I, P, P, I, I, L, P, P, I, I, F, P],
     "pylon_residual_add": [P, P, I, L, P],
-    "pylon_silu_gate": [P, P, I, I, I, P],
+    "pylon_silu_gate": [P, I, P, I, I, I, P],
     "pylon_qkv_prepare": [P, P, P, P, I, L, P, P, F, P, I, P, P, I, I, I, I, I, P],
     "pylon_paged_attention": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, P],
     "pylon_attention_decode": [P, P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, L, P],

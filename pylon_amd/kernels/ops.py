@@ -121,17 +121,20 @@ def residual_add(resid: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     return resid
 
 
-def silu_gate(gate_up: torch.Tensor, *, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``silu(gate_up[:, :I]) * gate_up[:, I:]`` for a ``[tokens, 2I]`` input."""
+def silu_gate(gate_up: torch.Tensor, *, out_dtype: Optional[torch.dtype] = None,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``silu(gate_up[:, :I]) * gate_up[:, I:]`` for a ``[tokens, 2I]`` input; the result may
+    have another element type than the input (float32 sums in, bfloat16 out: one rounding)."""
     if gate_up.dim() != 2 or gate_up.shape[1] % 2:
         raise KernelError("silu_gate takes a [tokens, 2*I] input")
     tokens, two_i = gate_up.shape
     inter = two_i // 2
+    out_dtype = out_dtype or (out.dtype if out is not None else gate_up.dtype)
     if out is None:
-        out = torch.empty((tokens, inter), dtype=gate_up.dtype, device=gate_up.device)
-    elif out.shape != (tokens, inter) or out.dtype != gate_up.dtype:
+        out = torch.empty((tokens, inter), dtype=out_dtype, device=gate_up.device)
+    elif out.shape != (tokens, inter) or out.dtype != out_dtype:
         raise KernelError("silu_gate: out has the wrong shape or dtype")
-    _lib.call("pylon_silu_gate", _dev(out, "out"), _dev(gate_up, "gate_up"),
+    _lib.call("pylon_silu_gate", _dev(out, "out"), dtype_code(out.dtype), _dev(gate_up, "gate_up"),
               dtype_code(gate_up.dtype), tokens, inter, _stream())
     return out
 
@@ -224,6 +227,10 @@ def decode_splits(tokens: int, n_kv_heads: int, max_len: Optional[int]) -> int:
     few thousand waves.  ``max_len`` is the most keys a workgroup gets (an upper bound
     under graph capture)."""
     waves = 8
+    if tokens * n_kv_heads > 256:
+        # more workgroups than compute units: smaller ones run side by side (64 tokens of 140
+        # keys: 13.8 us with four waves, 21.6 with eight; of 1,000 keys: 47 against 52)
+        waves = 4
     while waves > 1 and tokens * n_kv_heads * waves > 4096:
         waves //= 2
     if max_len is not None:
@@ -495,29 +502,23 @@ def k_parts(n: int, k: int) -> int:
 STREAM_ROWS = 64  # most rows of x one launch of the weight-streaming kernel takes
 
 
-def _streamed_float(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``x @ weight.T`` as unrounded float32 sums for any number of bfloat16 rows: the
-    weight-streaming kernel over groups of at most 64 rows (it re-reads ``weight`` once per
-    group)."""
-    if x.shape[0] <= STREAM_ROWS:
-        return gemm_skinny(x, weight, out_dtype=torch.float32, out=out)
+def _library_float(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x @ weight.T`` of bfloat16 operands as float32: the library's product with a float32
+    result, that is its float32 sums before any rounding."""
     if out is None:
-        out = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.float32, device=x.device)
-    for start in range(0, x.shape[0], STREAM_ROWS):
-        gemm_skinny(x[start: start + STREAM_ROWS], weight, out_dtype=torch.float32,
-                    out=out[start: start + STREAM_ROWS])
-    return out
+        return torch.mm(x, weight.t(), out_dtype=torch.float32)
+    return torch.mm(x, weight.t(), out_dtype=torch.float32, out=out)
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.dtype] = None,
            out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ weight.T`` (into ``out`` if given: contiguous, of the result's shape and type).
 
-    bfloat16 by bfloat16 with a bfloat16 result: up to 16 rows go to the weight-streaming
-    kernel, more rows to the library matrix product (as the reference's ``nn.Linear``
-    does); either way float32 sums are rounded once.  With a float32 result (the logits)
-    the sums come back unrounded whatever the number of rows, from the streaming kernel:
-    what a request's logits are rounded to does not depend on how many rows share its step.
+    bfloat16 by bfloat16: up to 16 rows go to the weight-streaming kernel, more rows to the
+    library matrix product (as the reference's ``nn.Linear`` does).  With a bfloat16 result
+    the float32 sums are rounded once either way; with a float32 result (the logits) they
+    come back unrounded either way (the library then writes its float32 sums): what a
+    request's logits are rounded to does not depend on how many rows share its step.
     Every pairing that involves float32 operands runs on the exact tiled kernel, which never
     uses a reduced-precision matrix mode.
     """
@@ -527,8 +528,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.d
             raise KernelError("linear: operands must live on the GPU; there is no CPU path")
         if skinny_ok(x, weight):
             return gemm_skinny(x, weight, out_dtype=out_dtype, out=out)
-        if out_dtype == torch.float32 and _streaming_ok(x, weight, 1 << 30):
-            return _streamed_float(x, weight, out)
+        if out_dtype == torch.float32:
+            return _library_float(x, weight, out)
         y = torch.nn.functional.linear(x, weight)
         y = y if out_dtype == torch.bfloat16 else y.to(out_dtype)
         return y if out is None else out.copy_(y)
@@ -537,21 +538,39 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.d
 
 def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:
     """A product whose result is about to be added to the float32 residual stream.  For up
-    to 64 bfloat16 rows it comes back as unrounded float32 partial sums ``[parts, M, N]``,
-    which the fused residual norm adds; for more rows (prompt portions) it is the library's
-    product, rounded once to bfloat16."""
+    to 64 bfloat16 rows it comes back as unrounded float32 sums, which the fused residual norm
+    adds: partial sums ``[parts, M, N]`` of the streaming kernel (K cut over workgroups), or,
+    for 17 to 64 rows of a matrix at which the library is faster, the library's float32
+    result.  For more rows (prompt portions) it is the library's product rounded once to
+    bfloat16."""
     if skinny_ok(x, weight):
         return gemm_skinny(x, weight, out_dtype=out_dtype, parts=k_parts(*weight.shape))
     if _streaming_ok(x, weight, STREAM_ROWS):
         n, k = weight.shape
-        return gemm_skinny(x, weight, out_dtype=out_dtype, parts=8 if k >= 16384 else 4, row_tiles=4)
+        if deep_or_small(n, k):
+            return gemm_skinny(x, weight, out_dtype=out_dtype, parts=8 if k >= 16384 else 4, row_tiles=4)
+        return _library_float(x, weight)
     return linear(x, weight, out_dtype=out_dtype)
 
 
+def deep_or_small(n: int, k: int) -> bool:
+    """Shapes at which, for 17 to 64 rows, the streaming kernel with K cut into parts beats
+    the library product: matrices much deeper than wide (a down projection; the library does
+    not cut K) and small ones (an out projection of a 4B or 8B model).  Measured at 64 rows:
+    2560x4096 14 against 19 us, 2560x9728 25 against 28, 4096x12288 32 against 37,
+    5120x25600 85 against 157; but 5120x8192 34 against 29, which stays with the library."""
+    return k >= 2 * n or n * k <= 24 * 1024 * 1024
+
+
 def linear_glu(x: torch.Tensor, gate_up: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:
-    """``silu(x @ gate.T) * (x @ up.T)`` for a fused ``[2I, K]`` gate/up matrix."""
+    """``silu(x @ gate.T) * (x @ up.T)`` for a fused ``[2I, K]`` gate/up matrix.  Up to 64
+    bfloat16 rows: the activation works on the float32 sums and its result is rounded once
+    (in the streaming kernel's epilogue up to 16 rows; from the library's float32 result up
+    to 64).  More rows (prompt portions): the library's product rounded to bfloat16 first."""
     if skinny_ok(x, gate_up):
         return gemm_skinny(x, gate_up, out_dtype=out_dtype, glu=True)
+    if x.dtype == torch.bfloat16 and gate_up.dtype == torch.bfloat16 and x.shape[0] <= STREAM_ROWS and x.is_cuda:
+        return silu_gate(_library_float(x, gate_up), out_dtype=out_dtype)
     return silu_gate(linear(x, gate_up, out_dtype=out_dtype))
 
 

@@ -738,3 +738,38 @@ def test_kernels_refuse_what_they_cannot_do(ops):
         ops.rmsnorm(torch.zeros((2, 8), dtype=torch.float16, device=DEV), torch.ones(8, device=DEV), 1e-6)
     with pytest.raises(KernelError, match="cannot multiply"):
         ops.gemm_tiled(torch.zeros((2, 8), device=DEV), torch.zeros((4, 9), device=DEV))
+
+
+def test_products_have_one_precision_at_every_row_count(ops):
+    """What a row's product is rounded to must not depend on how many rows share the call: the
+    logits (float32 result) and the products added to the residual stream are float32 sums
+    that were never rounded, from the weight-streaming kernel up to 16 rows and with the
+    library taking part beyond; the gated activation works on float32 sums and is rounded
+    once.  Rows of different calls then agree to float32 accuracy (the activation: up to rare
+    flips by one bfloat16 unit where a sum sits on a rounding boundary)."""
+    gen = torch.Generator().manual_seed(5)
+    k, inter = 2560, 1280
+    x = torch.randn((64, k), generator=gen).to(torch.bfloat16).to(DEV)
+    head = (torch.randn((3001, k), generator=gen) * 0.02).to(torch.bfloat16).to(DEV)
+    down = (torch.randn((k, 5120), generator=gen) * 0.02).to(torch.bfloat16).to(DEV)
+    wide = torch.randn((64, 5120), generator=gen).to(torch.bfloat16).to(DEV)
+    gate_up = (torch.randn((2 * inter, k), generator=gen) * 0.02).to(torch.bfloat16).to(DEV)
+    ref_head = x[0].double() @ head.double().T
+    ref_down = wide[0].double() @ down.double().T
+    gu = x[0].double() @ gate_up.double().T
+    ref_act = torch.nn.functional.silu(gu[:inter]) * gu[inter:]
+    acts = []
+    for rows in (1, 16, 17, 33, 64):
+        logits = ops.linear(x[:rows].contiguous(), head, out_dtype=torch.float32)
+        assert logits.dtype == torch.float32
+        assert float((logits[0].double() - ref_head).abs().max()) <= 2e-6 * float(ref_head.abs().max()), rows
+        delta = ops.linear_for_residual(wide[:rows].contiguous(), down, out_dtype=torch.bfloat16)
+        assert delta.dtype == torch.float32
+        total = delta.sum(dim=0) if delta.dim() == 3 else delta
+        assert float((total[0].double() - ref_down).abs().max()) <= 2e-6 * float(ref_down.abs().max()), rows
+        act = ops.linear_glu(x[:rows].contiguous(), gate_up, out_dtype=torch.bfloat16)
+        assert float((act[0].double() - ref_act).abs().max()) <= 2.0 ** -8 * float(ref_act.abs().max()), rows
+        acts.append(act[0].float())
+    for other in acts[1:]:
+        assert float((other != acts[0]).float().mean()) <= 5e-3  # one rounding each: they differ by rare flips only
+        assert float((other - acts[0]).abs().max()) <= 2.0 ** -7 * float(acts[0].abs().max())

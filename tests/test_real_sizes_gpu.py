@@ -123,3 +123,50 @@ def test_a_layer_of_the_widest_shape(tmp_path):
         got = np.concatenate([first[at: at + n], np.stack([rows[t][i] for t in range(decoded)])])
         at += n
         assert rows_within(got, ref, 3e-2)[0], (i, rows_within(got, ref, 3e-2))
+
+
+def test_logits_do_not_depend_on_how_many_requests_share_a_step(real):
+    """The same request decoded alone, as one of 16, of 20 and of 64: up to 16 rows every
+    product runs on the weight-streaming kernel, beyond that the library takes part.  Either
+    way the logits are float32 sums that were never rounded to bfloat16, the residual deltas
+    are float32 sums, and the activation is rounded once: what differs is the order of the
+    additions.  Up to 16 rows that order is the same, and the logits agree to the bit.  Beyond,
+    a float32 sum that lands on the other side of a bfloat16 rounding boundary flips a few
+    activations by one unit in the last place (3 of 6,144 in the q/k/v projection measured),
+    and the layers that follow amplify that (a flipped query element moved the feed-forward's
+    output by 1.4e-3 of its scale): the logits then agree within the bound that holds between
+    any two cuttings of the same work, and the greedy tokens are the same.  A head that rounds
+    to bfloat16 for more than 16 rows fails: its logits would all be bfloat16 numbers."""
+    from pylon_amd.engine import Runner, StepEntry
+
+    folder, cfg, _, _ = real
+    _, weights = read_folder(folder)
+    vocab = cfg["vocab_size"]
+    target = random_tokens(vocab, 23, 4242)
+    decoded = 6
+    others = [random_tokens(vocab, 4 + i % 9, 5000 + i) for i in range(63)]
+    want = plain.forward(weights, cfg, target)[-decoded:]
+    rows = {}
+    for batch in (1, 2, 16, 20, 64):
+        runner = Runner.from_folder(folder, dtype="bfloat16", page_size=256, num_pages=batch, max_requests=batch)
+        runner.enable_graphs(batch)
+        seqs = [runner.open(f"b{i}") for i in range(batch)]
+        prompts = [target[:-decoded]] + others[: batch - 1]
+        for seq, prompt in zip(seqs, prompts):  # every prompt alone: the same cache whatever the batch
+            runner.step([StepEntry(seq, prompt, [])])
+        got = []
+        for t in range(decoded):
+            entries = [StepEntry(seqs[0], [target[len(target) - decoded + t]], [0])]
+            entries += [StepEntry(s, [(7 * i + t) % vocab], [0]) for i, s in enumerate(seqs[1:])]
+            got.append(runner.step(entries)[0].cpu().numpy().copy())
+        assert runner.graphs.replays == decoded
+        rows[batch] = np.stack(got)
+        assert rows_within(rows[batch], want, 3e-2)[0], (batch, rows_within(rows[batch], want, 3e-2))
+        as_bf16 = torch.from_numpy(rows[batch]).to(torch.bfloat16).float().numpy()
+        assert (as_bf16 != rows[batch]).mean() > 0.5, f"batch {batch}: the logits were rounded to bfloat16"
+    for batch in (2, 16):
+        assert np.array_equal(rows[batch], rows[1]), f"batch {batch} differs from batch 1"
+    for batch in (20, 64):
+        ok, row, frac = rows_within(rows[batch], rows[1], 1e-2)
+        assert ok, f"batch {batch} differs from batch 1 at decoded token {row} by {frac:.2e} of its largest logit"
+        assert (rows[batch].argmax(axis=1) == rows[1].argmax(axis=1)).all(), batch
