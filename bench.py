@@ -257,6 +257,36 @@ def engine_run(runner, cfg, batch: int, seed: int, prompt_len: int = PROMPT_LEN,
     return batch * new_tokens / elapsed, 1e3 * first[len(first) // 2]
 
 
+def measured_peaks() -> dict:
+    """What this very device reaches on the two resources the fractions are priced against:
+    reading memory (this repository's streaming read kernel over 2 GiB, larger than every
+    cache) and bfloat16 matrix products (the library's product of 8,192-sized squares)."""
+    import torch
+
+    from pylon_amd.kernels import ops
+
+    data = torch.empty(1 << 29, dtype=torch.int32, device="cuda:0").fill_(1)
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda:0")
+
+    def timed(fn, repeats):
+        fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(repeats):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) * 1e-3 / repeats
+
+    read = data.numel() * 4 / timed(lambda: ops.probe_read(data, sink), 10)
+    del data
+    a = torch.randn(8192, 8192, device="cuda:0", dtype=torch.bfloat16)
+    b = torch.randn(8192, 8192, device="cuda:0", dtype=torch.bfloat16)
+    flops = 2.0 * 8192 ** 3 / timed(lambda: torch.mm(a, b.t()), 10)
+    return {"hbm_read_gbs": round(read / 1e9, 1), "bf16_gemm_tflops": round(flops / 1e12, 1)}
+
+
 def main() -> int:
     parser = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     parser.add_argument("--gpus", type=int, default=1)
@@ -270,6 +300,7 @@ def main() -> int:
     parser.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     parser.add_argument("--no-prefill", action="store_true")
+    parser.add_argument("--no-peaks", action="store_true", help="skip the probes of this device's own peaks")
     parser.add_argument("--mixed", action="store_true",
                         help="also time a step of --batch decoded tokens beside a 2,048-token prompt portion")
     parser.add_argument("--prefill-only", action="store_true",
@@ -342,6 +373,13 @@ def main() -> int:
         record["prefill"] = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
                              "ms": round(1e3 * seconds, 3),
                              "frac": round(flops / seconds / PEAK_FLOPS[dtype_key], 4)}
+    if not args.no_peaks:
+        peaks = measured_peaks()
+        record["measured_peaks"] = peaks
+        record["roofline"]["frac_of_measured"] = round(achieved / 1e9 / peaks["hbm_read_gbs"], 4)
+        if "prefill" in record and dtype_key == "bf16":
+            record["prefill"]["frac_of_measured"] = round(
+                record["prefill"]["frac"] * PEAK_FLOPS[dtype_key] / 1e12 / peaks["bf16_gemm_tflops"], 4)
     if args.mixed:
         seconds = mixed_run(runner, cfg, args.batch, prompt_len, repeats=5, seed=4)
         record["mixed"] = {"decodes": args.batch, "chunk": PREFILL_TOKENS, "ms": round(1e3 * seconds, 3)}

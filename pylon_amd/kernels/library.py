@@ -39,6 +39,7 @@ _SIGNATURES = {
     "pylon_gemm_skinny": [P, I, P, P, I, I, I, L, L, L, I, L, I, I, P],
     "pylon_argmax": [P, P, I, I, L, P, P, P, L, P],
     "pylon_argmax_static": [P, P, I, I, L, P, P, P],
+    "pylon_probe_read": [P, L, P, P],
     "pylon_sample": [P, P, I, I, L, P, P, P, P, P, P],
 }
 

@@ -630,3 +630,11 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
               _dev(temperature, "temperature", torch.float32), _dev(top_p, "top_p", torch.float32),
               _dev(uniform, "uniform", torch.float32), chosen_ptr, place_ptr, _stream())
     return out
+
+
+def probe_read(data: torch.Tensor, sink: torch.Tensor) -> None:
+    """Read every byte of ``data`` once (a measurement aid: the device's read bandwidth)."""
+    if not data.is_contiguous() or not data.is_cuda:
+        raise KernelError("probe_read takes a contiguous tensor on the GPU")
+    _lib.call("pylon_probe_read", data.data_ptr(), data.numel() * data.element_size(),
+              _dev(sink, "sink", torch.int32), _stream())
