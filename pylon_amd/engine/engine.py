@@ -164,6 +164,7 @@ class Engine:
         self._active: List[Active] = []
         self._lock = threading.RLock()
         self._wake = threading.Condition(self._lock)
+        self._ticking = threading.Lock()  # one tick at a time
         self._closed = False
         self.head_skips = 0
         self._serial = 0
@@ -287,24 +288,44 @@ class Engine:
 
     # ---- one tick ---------------------------------------------------------------------------
     def tick(self) -> bool:
-        """One round of admit, step, sample, finish.  True while work remains."""
-        with self._lock:
-            if self._closed:
-                return False
-            self._drop_cancelled_active()
-            self._admit()
-            try:
-                flight = self._launch_step() if self._active else None
-                if self._run_ahead:
-                    # The step just queued runs behind the one before it; now read that one.
-                    flight, self._flight = self._flight, flight
-                if flight is not None:
-                    self._land(flight)
-            except Exception as error:
-                logger.exception("model_batch_failed")
-                self._fail_active(error)
-            self._admit()
-            return bool(self._active or self._waiting or self._flight)
+        """One round of admit, step, sample, finish.  True while work remains.
+
+        The engine's lock guards its queue and its lists of requests, not the device: the one
+        place where a tick waits for the device, reading a step's sampled tokens, happens
+        with the lock released, so that ``enqueue``, ``snapshot`` and ``close`` from other
+        threads never wait for a step.  Ticks themselves run one at a time."""
+        with self._ticking:
+            with self._lock:
+                if self._closed:
+                    return False
+                self._drop_cancelled_active()
+                self._admit()
+                flight = None
+                try:
+                    flight = self._launch_step() if self._active else None
+                    if self._run_ahead:
+                        # The step just queued runs behind the one before it; now read that one.
+                        flight, self._flight = self._flight, flight
+                except Exception as error:
+                    logger.exception("model_batch_failed")
+                    self._fail_active(error)
+                    flight = None
+            token_ids, failure = [], None
+            if flight is not None and flight.draw is not None:
+                try:
+                    token_ids = flight.draw.result()  # waits for the device
+                except Exception as error:  # noqa: BLE001 - reported under the lock below
+                    failure = error
+            with self._lock:
+                if self._closed:
+                    return False
+                if failure is not None:
+                    logger.error("model_batch_failed: %s", failure)
+                    self._fail_active(failure)
+                elif flight is not None:
+                    self._land(flight, token_ids)
+                self._admit()
+                return bool(self._active or self._waiting or self._flight)
 
     # ---- admission ----------------------------------------------------------------------------
     def _sweep_cancelled_waiting(self) -> None:
@@ -402,6 +423,8 @@ class Engine:
                                            place=self.runner.logit_slots)
                 for item in ready:
                     item.awaiting = True
+            elif hasattr(self.sampler, "launch"):
+                draw = self.sampler.launch(logits, rows)  # read outside the lock, by tick
             else:
                 draw = _Drawn(self.sampler.sample(logits, rows))
             for item in ready:
@@ -410,9 +433,8 @@ class Engine:
             self.runner.synchronize()
         return Flight(draw, ready, decoding, portions, started)
 
-    def _land(self, flight: Flight) -> None:
-        """Read a step's tokens; finish or continue its requests."""
-        token_ids = flight.draw.result() if flight.draw is not None else []
+    def _land(self, flight: Flight, token_ids: Sequence[int]) -> None:
+        """A step's tokens have been read: finish or continue its requests."""
         sampled_at = self._clock()
         elapsed = sampled_at - max(flight.started, self._landed_at)
         self._landed_at = sampled_at

@@ -38,6 +38,20 @@ def margins_ok(weights, cfg, prompt, produced, floor):
     return True
 
 
+def follows_plain(weights, cfg, prompt, produced, slack):
+    """Every produced token is the plain model's greedy choice given the tokens before it (the
+    produced ones, so that one flipped near-tie does not excuse what follows), or loses to
+    that choice by no more than ``slack`` times the row's largest |logit|.  Returns the index
+    of the first token that is neither, or None."""
+    tokens = list(prompt)
+    for i, tok in enumerate(produced):
+        row = plain.forward(weights, cfg, tokens)[-1]
+        if tok != int(row.argmax()) and row.max() - row[tok] > slack * np.abs(row).max():
+            return i
+        tokens.append(tok)
+    return None
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_greedy_generation_through_the_engine(tmp, dtype):
     """Tiny A's workload: prompts of 5, 17 and 33 tokens, 16 greedy tokens each, all three
@@ -61,10 +75,39 @@ def test_greedy_generation_through_the_engine(tmp, dtype):
         if dtype == "float32":
             assert result.output_ids == want
         else:
-            # bfloat16 may flip a near-tie; up to the first flip the tokens must agree,
-            # and a flip is only allowed where the plain model's margin is small
+            # bfloat16 may flip a near-tie: every token, given the engine's own tokens before
+            # it, must be the plain model's choice or within the logits' error bound of it
+            assert follows_plain(weights, cfg, prompt, result.output_ids, 2e-2) is None
             agree = next((i for i, (a, b) in enumerate(zip(result.output_ids, want)) if a != b), 16)
             assert agree == 16 or not margins_ok(weights, cfg, prompt, want[: agree + 1], 0.02)
+
+
+def test_the_threaded_engine_on_the_gpu(tmp):
+    """The background thread drives the real step function while requests arrive from this
+    thread; results are the plain model's greedy tokens (float32: exactly)."""
+    import time
+
+    from pylon_amd.engine.engine import Engine
+    from pylon_amd.sampling import Sampling
+
+    folder = make_model_folder(tmp, "B", dtype="float32", std=0.08)
+    cfg, weights = read_folder(folder)
+    prompts = [random_tokens(cfg["vocab_size"], n, 300 + n) for n in (3, 40, 9, 21, 2, 65)]
+    engine = Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=40, max_batch_size=3,
+                                prefill_chunk_size=16, threaded=True)
+    try:
+        futures = []
+        for prompt in prompts:
+            futures.append(engine.enqueue(prompt, None, Sampling(max_new_tokens=6, temperature=0.0)))
+            time.sleep(0.002)  # arrivals spread over the ticks
+            assert set(engine.snapshot()) >= {"waiting", "active"}
+        results = [f.result(timeout=60) for f in futures]
+    finally:
+        engine.close()
+    for prompt, result in zip(prompts, results):
+        assert result.output_ids == plain_generate(weights, cfg, prompt, 6, lambda row, i: plain.greedy(row))
+        assert result.first_token_seconds is not None and len(result.token_intervals) == 5
+    assert engine.runner.manager.free_pages == 40
 
 
 def test_stop_token_and_first_token_from_a_one_token_prompt(tmp):

@@ -551,3 +551,47 @@ def test_results_carry_the_reference_timing_fields():
     assert len(result.output_ids) == 4 and len(result.token_intervals) == 3
     assert result.first_token_at == pytest.approx(1000.0 + result.first_token_seconds)
     assert all(abs(dt - 0.25) < 1e-9 for dt in result.token_intervals)
+
+
+def test_enqueue_and_snapshot_do_not_wait_for_a_step():
+    """A tick waits for the device only while it reads a step's tokens, and it holds no lock
+    then: a request arrives, and the engine's state can be read, while that wait lasts."""
+    import threading
+
+    release, waiting = threading.Event(), threading.Event()
+
+    class SlowSampler(ScriptedSampler):
+        def launch(self, logits, rows, **_):
+            ids = self.sample(logits, rows)
+
+            class Draw:
+                def result(self):
+                    waiting.set()
+                    assert release.wait(10)
+                    return ids
+
+            return Draw()
+
+    config = PylonConfig(max_batch_size=4, page_size=PAGE, run_ahead=False)
+    engine = Engine(config, runner=FakeRunner(8), sampler=SlowSampler(), clock=Clock())
+    first = enqueue(engine, "first", [1, 2, 3], 2)
+    ticker = threading.Thread(target=engine.tick)
+    ticker.start()
+    try:
+        assert waiting.wait(10)  # the tick is inside its wait for the device
+        done = threading.Event()
+        box = {}
+
+        def arrive():
+            box["future"] = enqueue(engine, "second", [4, 5], 1)
+            box["snapshot"] = engine.snapshot()
+            done.set()
+
+        threading.Thread(target=arrive).start()
+        assert done.wait(2), "enqueue waited for the step"
+        assert box["snapshot"]["waiting"] == ["second"] and box["snapshot"]["active"] == ["first"]
+    finally:
+        release.set()
+        ticker.join(10)
+    engine.run_until_idle()
+    assert first.result(timeout=1).output_ids == [7, 7] and box["future"].result(timeout=1).output_ids == [7]
