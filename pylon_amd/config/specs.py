@@ -116,6 +116,11 @@ class ModelSpec:
     tie_word_embeddings: bool
     max_positions: int
     embedding_scale: float = 1.0
+    # Parts between the embedding and the first layer (family "stream": an embedding norm,
+    # learned positions, ...) and parts after the vocabulary head (family "logits": a soft
+    # cap, a scale, ...), as specs with a ``kind``; the Qwen3 decoder has neither.
+    stream_parts: Tuple[object, ...] = ()
+    logit_parts: Tuple[object, ...] = ()
     extra: dict = field(default_factory=dict, compare=False, hash=False)
 
     def resolved_schedule(self) -> Tuple[Tuple[int, int, bool], ...]:

@@ -3,7 +3,11 @@
 The model is architecture-blind: it builds one block per :class:`LayerSpec`, runs the
 blocks in the order the schedule lists them, and applies the final norm and the
 vocabulary head only at the tokens whose logits are wanted
-(/root/reference/src/pylon/model/model.py:124-144).
+(/root/reference/src/pylon/model/model.py:124-144).  What an architecture does outside
+its layers goes into two optional lists of parts: "stream" parts between the embedding and
+the first layer (``forward(resid, ctx) -> resid``, the float32 residual stream of the step's
+tokens), "logits" parts after the head (``forward(logits, ctx) -> logits``, float32, one row
+per wanted token; under graph replay they must write in place).
 """
 from __future__ import annotations
 
@@ -38,6 +42,10 @@ class Model(Part):
         self.final_norm = self.add_child(
             "final_norm", build_part("norm", spec.final_norm, dtype=dtype, device=device)
         )
+        self.stream_parts = [self.add_child(f"stream.{i}", build_part("stream", part, dtype=dtype, device=device))
+                             for i, part in enumerate(spec.stream_parts)]
+        self.logit_parts = [self.add_child(f"logits.{i}", build_part("logits", part, dtype=dtype, device=device))
+                            for i, part in enumerate(spec.logit_parts)]
 
     # ---- what the cache manager has to provide ------------------------------------------
     def cache_requirements(self) -> List[object]:
@@ -64,6 +72,8 @@ class Model(Part):
         Returns float32 logits ``[n_logits, vocab]`` (None when no logits are wanted)."""
         resid = ops.embed(ctx.token_ids, self.params["embed"], scale=self.spec.embedding_scale,
                           chosen=ctx.chosen)
+        for part in self.stream_parts:
+            resid = part.forward(resid, ctx)
         delta = None
         for layer, cache_id, stores in self.schedule:
             resid, delta = self.blocks[layer].forward(resid, delta, ctx, ctx.cache(cache_id), stores)
@@ -71,4 +81,7 @@ class Model(Part):
             return None
         h = self.final_norm.add_forward(resid, delta, row_idx=ctx.logit_idx)
         out = None if ctx.logits_out is None else ctx.logits_out[: ctx.n_logits]
-        return ops.linear(h, self.head_weight, out_dtype=torch.float32, out=out)
+        logits = ops.linear(h, self.head_weight, out_dtype=torch.float32, out=out)
+        for part in self.logit_parts:
+            logits = part.forward(logits, ctx)  # in place where ``out`` was given
+        return logits

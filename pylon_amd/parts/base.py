@@ -23,6 +23,11 @@ mixer         ``cache_requirement() -> KVRequirement | StateRequirement | None``
 feed_forward  ``forward(h, ctx) -> [tokens, hidden]``.
 block         ``forward(resid, delta, ctx, cache, stores) -> (resid, delta)``: takes and
               returns the residual stream and the not-yet-added output of the last part.
+stream        ``forward(resid, ctx) -> resid``: the embedded tokens (float32 ``[tokens, dim]``)
+              before the first layer: an embedding norm, learned positions
+              (``ctx.positions``), a scale.
+logits        ``forward(logits, ctx) -> logits``: float32 ``[wanted, vocab]`` after the
+              vocabulary head: a soft cap, a scale, a bias (in place).
 """
 from __future__ import annotations
 

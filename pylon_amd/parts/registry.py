@@ -2,13 +2,15 @@
 
 A model is put together by looking up each spec of a :class:`LayerSpec` here, so a new
 mixer, feed-forward, norm, position encoding or block arrangement is added by
-registering a class; no file of the framework has to change.
+registering a class; no file of the framework has to change.  Two more families hold what
+a model may do outside its layers: "stream" parts work on the embedded tokens before the
+first layer, "logits" parts on the logits after the vocabulary head.
 """
 from __future__ import annotations
 
 from typing import Callable, Dict
 
-_FAMILIES = ("mixer", "feed_forward", "norm", "position", "block")
+_FAMILIES = ("mixer", "feed_forward", "norm", "position", "block", "stream", "logits")
 _PARTS: Dict[str, Dict[str, Callable]] = {family: {} for family in _FAMILIES}
 
 
