@@ -3,9 +3,7 @@
 //
 // A workgroup of 4 or 8 wavefronts owns 16 rows of w (16 output columns), or 32 rows as two
 // tiles for matrices with many rows (the rows of x it loads then serve both; measured
-// 151 us against 165 us for a 151936 x 2560 matrix), or, on request, 64 rows as four tiles
-// (for 17 to 64 rows of x, which are two to four tiles themselves and would else be most of
-// what a workgroup reads).  The waves take
+// 151 us against 165 us for a 151936 x 2560 matrix).  The waves take
 // turns along K in steps of 64: in a step a wave reads one full 128-byte line of each of
 // its 16 rows, as two loads that each cover a contiguous 64-byte half of every line.
 // All loads of a batch of steps are issued before the first product, so a wave with few
@@ -169,19 +167,12 @@ static void launch_skinny(void* out, int out_dtype, const void* x, const void* w
 template <int MT>
 static void launch_skinny_mt(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                              long long ldx, long long ldw, long long ldo, int parts,
-                             long long part_stride, int glu, int row_tiles, hipStream_t stream) {
+                             long long part_stride, int glu, hipStream_t stream) {
   // Four waves measured faster than eight at every shape of a 4B-class decoder; the
   // eight-wave form is kept for very long K only.
   const int steps = (K + SK_STEP - 1) / SK_STEP / parts;
   const bool wide = steps >= 512;
 #define GO(W, G, R) launch_skinny<MT, W, G, R>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream)
-  if constexpr (MT > 1) {
-    // Several tiles of x: four tiles of w share them if the caller asks for it.
-    if (row_tiles == 4 && !glu) {
-      GO(4, false, 4);
-      return;
-    }
-  }
   if (glu) {
     if (wide) GO(8, true, 1); else GO(4, true, 1);
   } else if (MT == 1 && parts == 1 && N >= 4096) {
@@ -199,10 +190,8 @@ static void launch_skinny_mt(void* out, int out_dtype, const void* x, const void
 // and no glu).
 extern "C" int pylon_gemm_skinny(void* out, int out_dtype, const void* x, const void* w, int M, int N,
                                  int K, long long ldx, long long ldw, long long ldo, int parts,
-                                 long long part_stride, int glu, int row_tiles, hipStream_t stream) {
+                                 long long part_stride, int glu, hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(out_dtype), "gemm_skinny: unknown output dtype");
-  PYLON_REQUIRE(row_tiles == 0 || (row_tiles == 4 && !glu),
-                "gemm_skinny: row_tiles is 0 (automatic) or, without glu, 4; got %d", row_tiles);
   PYLON_REQUIRE(M >= 0 && M <= 64, "gemm_skinny: takes at most 64 rows, got %d", M);
   PYLON_REQUIRE(N > 0 && K > 0, "gemm_skinny: bad sizes N=%d K=%d", N, K);
   PYLON_REQUIRE(K % 8 == 0, "gemm_skinny: K=%d must be a multiple of 8", K);
@@ -217,10 +206,10 @@ extern "C" int pylon_gemm_skinny(void* out, int out_dtype, const void* x, const 
                 "gemm_skinny: partial results overlap");
   if (M == 0) return 0;
   switch ((M + 15) / 16) {
-    case 1: launch_skinny_mt<1>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, row_tiles, stream); break;
-    case 2: launch_skinny_mt<2>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, row_tiles, stream); break;
-    case 3: launch_skinny_mt<3>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, row_tiles, stream); break;
-    default: launch_skinny_mt<4>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, row_tiles, stream); break;
+    case 1: launch_skinny_mt<1>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, stream); break;
+    case 2: launch_skinny_mt<2>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, stream); break;
+    case 3: launch_skinny_mt<3>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, stream); break;
+    default: launch_skinny_mt<4>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, glu, stream); break;
   }
   PYLON_LAUNCHED("gemm_skinny");
 }

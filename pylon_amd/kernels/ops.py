@@ -455,15 +455,13 @@ def skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
 
 
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype = torch.bfloat16,
-                parts: int = 1, glu: bool = False, row_tiles: int = 0,
+                parts: int = 1, glu: bool = False,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ weight.T`` for at most 64 rows of bfloat16 ``x``, streaming ``weight`` once.
 
     ``parts > 1`` cuts K into that many ranges and returns float32 partial results
     ``[parts, M, N]`` for the consumer to add.  ``glu``: ``weight`` is a fused
     ``[2N, K]`` gate/up matrix and the result is ``silu(x @ gate.T) * (x @ up.T)``.
-    ``row_tiles=4`` (more than 16 rows, no ``glu``): a workgroup takes 64 rows of ``weight``
-    instead of 16, so that the rows of ``x`` it reads serve four times as many.
     """
     if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
         raise KernelError(f"gemm_skinny: cannot multiply {tuple(x.shape)} by the transpose of {tuple(weight.shape)}")
@@ -484,7 +482,32 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype
             or not out.is_cuda or not out.is_contiguous():
         raise KernelError(f"gemm_skinny: out must be contiguous, on the GPU and of shape {shape}")
     _lib.call("pylon_gemm_skinny", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), weight.data_ptr(),
-              m, n, k, x.stride(0), weight.stride(0), n, parts, m * n, 1 if glu else 0, int(row_tiles), _stream())
+              m, n, k, x.stride(0), weight.stride(0), n, parts, m * n, 1 if glu else 0, _stream())
+    return out
+
+
+def gemm_rows(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype = torch.bfloat16,
+              parts: int = 1, col_tiles: int = 1, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x @ weight.T`` for at most 64 rows of bfloat16 ``x``, made for 17 to 64: the rows of
+    ``x`` pass through LDS once per workgroup of 64 (``col_tiles=1``) or 128 (``col_tiles=2``)
+    columns and ``weight`` is streamed once.  ``parts > 1`` cuts K into that many ranges and
+    returns float32 partial results ``[parts, M, N]`` for the consumer to add."""
+    if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
+        raise KernelError(f"gemm_rows: cannot multiply {tuple(x.shape)} by the transpose of {tuple(weight.shape)}")
+    m, k = x.shape
+    n = weight.shape[0]
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise KernelError("gemm_rows takes bfloat16 operands")
+    if not (x.is_cuda and weight.is_cuda) or x.stride(1) != 1 or weight.stride(1) != 1:
+        raise KernelError("gemm_rows: operands must be on the GPU with contiguous rows")
+    shape = (parts, m, n) if parts > 1 else (m, n)
+    if out is None:
+        out = torch.empty(shape, dtype=torch.float32 if parts > 1 else out_dtype, device=x.device)
+    elif tuple(out.shape) != shape or out.dtype != (torch.float32 if parts > 1 else out_dtype) \
+            or not out.is_cuda or not out.is_contiguous():
+        raise KernelError(f"gemm_rows: out must be contiguous, on the GPU and of shape {shape}")
+    _lib.call("pylon_gemm_rows", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), weight.data_ptr(),
+              m, n, k, x.stride(0), weight.stride(0), n, parts, m * n, int(col_tiles), _stream())
     return out
 
 
@@ -539,7 +562,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.d
 def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:
     """A product whose result is about to be added to the float32 residual stream.  For up
     to 64 bfloat16 rows it comes back as unrounded float32 sums, which the fused residual norm
-    adds: partial sums ``[parts, M, N]`` of the streaming kernel (K cut over workgroups), or,
+    adds: partial sums ``[parts, M, N]`` of a streaming kernel (K cut over workgroups), or,
     for 17 to 64 rows of a matrix at which the library is faster, the library's float32
     result.  For more rows (prompt portions) it is the library's product rounded once to
     bfloat16."""
@@ -548,18 +571,33 @@ def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: tor
     if _streaming_ok(x, weight, STREAM_ROWS):
         n, k = weight.shape
         if deep_or_small(n, k):
-            return gemm_skinny(x, weight, out_dtype=out_dtype, parts=8 if k >= 16384 else 4, row_tiles=4)
+            parts, col_tiles = rows_plan(n, k)
+            return gemm_rows(x, weight, out_dtype=torch.float32, parts=parts, col_tiles=col_tiles)
         return _library_float(x, weight)
     return linear(x, weight, out_dtype=out_dtype)
 
 
 def deep_or_small(n: int, k: int) -> bool:
-    """Shapes at which, for 17 to 64 rows, the streaming kernel with K cut into parts beats
-    the library product: matrices much deeper than wide (a down projection; the library does
-    not cut K) and small ones (an out projection of a 4B or 8B model).  Measured at 64 rows:
-    2560x4096 14 against 19 us, 2560x9728 25 against 28, 4096x12288 32 against 37,
-    5120x25600 85 against 157; but 5120x8192 34 against 29, which stays with the library."""
-    return k >= 2 * n or n * k <= 24 * 1024 * 1024
+    """Shapes at which, for 17 to 64 rows, the kernel that shares the rows of x through LDS
+    and cuts K into parts beats the library product: matrices much deeper than wide (a down
+    projection; the library does not cut K) and those of few rows (an out projection).
+    Measured at 64 rows: 2560x4096 11 against 14 us, 2560x9728 21 against 28, 4096x4096 12
+    against 15, 4096x12288 29 against 39, 5120x25600 79 against 90; but 5120x8192 30 against
+    29 and 8192x8192 39 against 35, which stay with the library."""
+    return k >= 2 * n or n <= 4096
+
+
+def rows_plan(n: int, k: int) -> tuple:
+    """(parts, col_tiles) for :func:`gemm_rows` on an ``[n, k]`` matrix: workgroups of 128
+    columns for deep matrices, else of 64, and K cut into the largest power of two of parts
+    (at most 16, of at least 256 elements each) that keeps the workgroups at 256 or fewer, one
+    per compute unit: more of them only re-read the rows of x."""
+    col_tiles = 2 if k >= 8192 else 1
+    groups = -(-n // (64 * col_tiles))
+    parts = 1
+    while parts < 16 and 2 * parts * groups <= 256 and k // (2 * parts) >= 256:
+        parts *= 2
+    return parts, col_tiles
 
 
 def linear_glu(x: torch.Tensor, gate_up: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:

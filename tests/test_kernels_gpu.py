@@ -193,14 +193,6 @@ def test_gemm_skinny(ops, shape):
         got = ops.gemm_skinny(a.to(DEV), w.to(DEV), parts=parts)
         assert got.shape == (parts, m, n) and got.dtype == torch.float32
         assert np.abs(f64(got).sum(0) - want).max() <= tol(torch.float32, np.abs(want).max())
-    if m > 16:  # four tiles of w to a workgroup, alone and with K cut
-        for parts in (1, 4, 8):
-            got = ops.gemm_skinny(a.to(DEV), w.to(DEV), out_dtype=torch.float32, parts=parts, row_tiles=4)
-            got = got.sum(0) if parts > 1 else got
-            assert got.shape == (m, n)
-            assert np.abs(f64(got) - want).max() <= tol(torch.float32, np.abs(want).max())
-        one = ops.gemm_skinny(a[5:6].contiguous().to(DEV), w.to(DEV), parts=4)
-        assert torch.equal(one[:, 0], ops.gemm_skinny(a.to(DEV), w.to(DEV), parts=4, row_tiles=4)[:, 5])
     # the same rows give the same bits whatever other rows share the launch
     full = ops.gemm_skinny(a.to(DEV), w.to(DEV), out_dtype=torch.float32)
     alone = ops.gemm_skinny(a[:1].contiguous().to(DEV), w.to(DEV), out_dtype=torch.float32)
@@ -227,6 +219,44 @@ def test_gemm_skinny(ops, shape):
     from pylon_amd.kernels import KernelError
     with pytest.raises(KernelError, match="at most 64 rows"):
         ops.gemm_skinny(torch.zeros((65, 64), dtype=torch.bfloat16, device=DEV), w[:, :64].contiguous().to(DEV))
+
+
+@pytest.mark.parametrize("shape", [(17, 100, 200), (64, 2560 + 8, 512 + 24), (33, 61, 136), (50, 333, 1000),
+                                   (64, 129, 128), (48, 64, 8), (20, 72, 9728), (1, 77, 264), (16, 300, 392)])
+def test_gemm_rows(ops, shape):
+    """The product for 17 to 64 rows (x shared through LDS, w streamed, three chunks in
+    flight): every size class (rows in 1 to 4 tiles, columns and K that end inside a tile or
+    a chunk, K shorter than a chunk), K cut into parts, both workgroup widths."""
+    m, n, k = shape
+    a, w = rnd((m, k), 32, torch.bfloat16), rnd((n, k), 33, torch.bfloat16, 0.1)
+    want = f64(a) @ f64(w).T
+    ref = None
+    for col_tiles in (1, 2):
+        for out_dtype in (torch.bfloat16, torch.float32):
+            got = ops.gemm_rows(a.to(DEV), w.to(DEV), out_dtype=out_dtype, col_tiles=col_tiles)
+            assert got.shape == (m, n) and got.dtype == out_dtype
+            assert np.abs(f64(got) - want).max() <= tol(out_dtype, np.abs(want).max())
+        # the two widths add in the same order
+        ref = got if ref is None else ref
+        assert torch.equal(ref, got)
+        for parts in (2, 3, 8, 16):
+            got = ops.gemm_rows(a.to(DEV), w.to(DEV), parts=parts, col_tiles=col_tiles)
+            assert got.shape == (parts, m, n) and got.dtype == torch.float32
+            assert np.abs(f64(got).sum(0) - want).max() <= tol(torch.float32, np.abs(want).max())
+    # the same rows give the same bits whatever other rows share the launch
+    full = ops.gemm_rows(a.to(DEV), w.to(DEV), parts=4)
+    alone = ops.gemm_rows(a[m // 2: m // 2 + 1].contiguous().to(DEV), w.to(DEV), parts=4)
+    assert torch.equal(alone[:, 0], full[:, m // 2])
+    with pytest.raises(Exception, match="at most 64 rows"):
+        ops.gemm_rows(rnd((65, k), 34, torch.bfloat16).to(DEV), w.to(DEV))
+
+
+def test_rows_plan_keeps_the_workgroups_within_the_chip(ops):
+    for n, k in [(2560, 4096), (2560, 9728), (4096, 12288), (5120, 25600), (1024, 2048), (64, 512), (100, 256)]:
+        parts, col_tiles = ops.rows_plan(n, k)
+        groups = -(-n // (64 * col_tiles))
+        assert col_tiles in (1, 2) and 1 <= parts <= 16
+        assert parts == 1 or (parts * groups <= 256 and k // parts >= 256)
 
 
 def plain_rope(x, pos, inv_freq, rot):
