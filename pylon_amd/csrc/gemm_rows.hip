@@ -6,215 +6,256 @@
 // tiles of 16 rows of w) over a range of K; K is cut over blockIdx.y and every cut writes
 // its own float partial result, which the consumer adds (the fused residual norm does), or,
 // with one cut, the result itself.  The workgroup walks its range in chunks of 128 elements.
-// The rows of x of a chunk go from memory straight into LDS (buffer_load_dwordx4 ... lds: a wave
-// fills 1 KB of consecutive LDS from 64 places of its choice, here the 16 rows x 4 pieces of
-// 16 bytes that are one column operand of the 16x16x32 matrix instruction, in lane order, so
-// that reading an operand back is one conflict-free 16-byte read per lane) and are shared by
-// the four waves; each wave loads its own tiles of w into registers in the layout of the
-// row operand.  Three chunks are in flight: while chunk c is multiplied, c + 1 and c + 2
-// travel.  There is one barrier per chunk, preceded by a counted wait for this wave's loads of
-// chunk c only, so the later loads stay in flight across it.  No sums cross waves: a wave owns its columns.
 //
-// All loads go through buffer descriptors (of the workgroup's rows of w; of x): rows beyond N
-// and elements beyond K are read as zeros without a memory access and without a branch, so
-// every wave issues the same number of loads per chunk and the counted waits below are exact.
+// Both operands travel from memory straight into LDS (buffer_load_dwordx4 ... lds: a wave
+// fills 1 KB of consecutive LDS from 64 places of its choice) in whole row segments: one
+// load takes the 256 contiguous bytes that a chunk is of each of four rows.  (A load that
+// takes 64 bytes of each of 16 rows, the shape of a matrix-instruction operand, moves less
+// than half as much per compute unit: measured 21 us against 8 us for the rows of x of a
+// 19456 x 2560 product.)  The rows of x of a chunk are shared by the four waves; each wave
+// brings its own tiles of w.  In LDS a tile is 16 rows of 256 bytes, and the 16-byte piece q
+// of row R lies at position q ^ R of that row, so that the operand reads (lane r takes piece
+// 4 s + g of row r) of 16 lanes fall into 16 different groups of banks.  Several chunks are in
+// flight: while chunk c is multiplied, the next two or three travel.  There is one barrier
+// per chunk, preceded by a counted wait for this wave's loads of chunk c only, so the later
+// loads stay in flight across it.  No sums cross waves: a wave owns its columns.
+//
+// All loads go through buffer descriptors (of the workgroup's rows of w; of x): rows beyond
+// N or M and elements beyond K are read as zeros without a memory access and without a
+// branch, so every wave issues the same number of loads per chunk and the counted waits
+// are exact.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef int intx4 __attribute__((ext_vector_type(4)));
 
 #define GR_CHUNK 128
-#define GR_STAGES 3
+#define GR_TILE_BYTES 4096  // 16 rows of one chunk
 #define GR_WAVES 4
-#define GR_GLOBAL(T) __attribute__((address_space(1))) T
 #define GR_LDS(T) __attribute__((address_space(3))) T
 #define GR_OOB 0x80000000u
-
 
 // A bare barrier: the waits that must precede it are counted by hand below.  (A release
 // fence on LDS would wait for every outstanding load, because the loads that write LDS are
 // among them, and the chunks in flight would drain at every barrier.)
 __device__ __forceinline__ void gr_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
-// vmcnt <= N (N < 16); the other counters are left alone.
+__device__ __forceinline__ float gr_silu(float z) { return z / (1.0f + expf(-z)); }
+
+// vmcnt <= N (N < 64); the other counters are left alone.
 template <int N>
 __device__ __forceinline__ void gr_wait_loads() {
-  static_assert(N >= 0 && N < 16, "vmcnt beyond the low field");
-  __builtin_amdgcn_s_waitcnt(0x0f70 | N);
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
 }
 
-// MT: tiles of 16 rows of x (2..4); CT: tiles of 16 rows of w per wave (1 or 2).
+// Stages of LDS for MT tiles of x and 4 * CT tiles of w per chunk: as many as fit, at most 4.
+template <int MT, int CT>
+struct GrShape {
+  static constexpr int TILES = MT + GR_WAVES * CT;
+  static constexpr int STAGE_BYTES = TILES * GR_TILE_BYTES;
+  static constexpr int STAGES = (4 * STAGE_BYTES <= 144 * 1024) ? 4 : 3;
+};
+
+// MT: tiles of 16 rows of x (1..4); CT: tiles of 16 rows of w per wave (1 or 2).
+// GLU (CT = 2): w is a fused gate/up matrix of 2 N rows; a wave's first tile is 16 gate rows,
+// its second the 16 up rows that lie N rows further down, and it writes silu(gate) * up.
 // (The body is a device function: the host pass does not know the descriptor type and would
 // drop a kernel that names it, launch stub and all.)
-template <int MT, int CT, typename TO>
+template <int MT, int CT, bool GLU, typename TO>
 __device__ __forceinline__ void gemm_rows_body(
     TO* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int M, int N,
     int K, long long ldx, long long ldw, long long ldo, long long part_stride, int chunks_per_part) {
-  constexpr int FRAGS = MT * 4;             // operands of x per chunk: tile t, step s -> 4 t + s
-  constexpr int XL = FRAGS / GR_WAVES;      // of which a wave fetches this many
-  constexpr int LOADS = XL + 4 * CT;        // loads a wave issues per chunk
-  static_assert(FRAGS % GR_WAVES == 0, "the waves share the operands of x evenly");
-  __shared__ __attribute__((aligned(1024))) unsigned char xs[GR_STAGES][FRAGS][1024];
+  typedef GrShape<MT, CT> Shape;
+  constexpr int STAGES = Shape::STAGES;
+  constexpr int LOADS = MT + 4 * CT;  // loads a wave issues per chunk
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * Shape::STAGE_BYTES];
 
   const int lane = threadIdx.x & (PYLON_WAVE - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PYLON_WAVE);
   const int r = lane & 15, g = lane >> 4;
-  const int wg_row0 = blockIdx.x * (GR_WAVES * CT * 16);  // first row of w of this workgroup
-  const int n0 = wg_row0 + wave * CT * 16;                // and of this wave
+  constexpr int WG_COLS = GR_WAVES * (GLU ? 1 : CT) * 16;  // columns of the output per workgroup
+  const int wg_row0 = blockIdx.x * WG_COLS;                // first row of w of this workgroup
+  const int n0 = wg_row0 + wave * (WG_COLS / GR_WAVES);    // and of this wave
   const int part = blockIdx.y;
   const int chunks = (K + GR_CHUNK - 1) / GR_CHUNK;
   const int c_begin = part * chunks_per_part;
   const int c_end = (c_begin + chunks_per_part < chunks) ? c_begin + chunks_per_part : chunks;
 
-  // w: a descriptor over this workgroup's rows, so that offsets fit 31 bits whatever N is.
-  const int wg_rows = (N - wg_row0 < GR_WAVES * CT * 16) ? N - wg_row0 : GR_WAVES * CT * 16;
+  // The descriptor of w starts at the workgroup's first row (with GLU it reaches N rows
+  // further, to its up rows: the host checks that this fits 31 bits).
+  const int wg_rows = (N - wg_row0 < WG_COLS) ? N - wg_row0 : WG_COLS;
   const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t*>(w + static_cast<size_t>(wg_row0) * ldw), 0,
-      static_cast<int>((static_cast<long long>(wg_rows - 1) * ldw + K) * 2), 0x00020000);
-  unsigned w_row[CT];  // byte offset of this lane's row in each tile, or out of range
-#pragma unroll
-  for (int j = 0; j < CT; ++j) {
-    const int row = wave * CT * 16 + 16 * j + r;
-    w_row[j] = (wg_row0 + row < N) ? static_cast<unsigned>(row) * static_cast<unsigned>(ldw) * 2u : GR_OOB;
-  }
-  // x: operand f = wave + 4 i of a chunk is fetched by this wave; its row and step.  Rows
-  // beyond M repeat the last one (their columns of the result are never stored).
+      static_cast<int>((static_cast<long long>((GLU ? N : 0) + wg_rows - 1) * ldw + K) * 2), 0x00020000);
   const __amdgpu_buffer_rsrc_t xres = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t*>(x), 0, static_cast<int>((static_cast<long long>(M - 1) * ldx + K) * 2), 0x00020000);
-  unsigned x_row[XL];
-  int x_step[XL];
-#pragma unroll
-  for (int i = 0; i < XL; ++i) {
-    const int f = wave + GR_WAVES * i, t = f >> 2;
-    const int m = (t * 16 + r < M) ? t * 16 + r : M - 1;
-    x_row[i] = static_cast<unsigned>(m) * static_cast<unsigned>(ldx) * 2u;
-    x_step[i] = (f & 3) * 32 + g * 8;
-  }
 
-  intx4 wreg[GR_STAGES][CT][4];
+  // A load fills rows 4 q .. 4 q + 3 of a tile (q: the quarter): lane l brings, for row
+  // R = 4 q + l / 16, the piece (l % 16) ^ R.
+  // x: this wave fills quarter `wave` of every tile of x.
+  const int lrow = lane >> 4, lpos = lane & 15;
+  unsigned x_at[MT];  // byte offset of this lane's piece in chunk 0, or out of range
+  int x_k;            // its first element within a chunk
+  {
+    const int R = 4 * wave + lrow;
+    x_k = (lpos ^ R) * 8;
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+      x_at[t] = (16 * t + R < M)
+                    ? static_cast<unsigned>(16 * t + R) * static_cast<unsigned>(ldx) * 2u + 2u * x_k
+                    : GR_OOB;
+  }
+  // w: this wave fills all four quarters of its own CT tiles.
+  unsigned w_at[CT][4];
+  int w_k[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int R = 4 * q + lrow;
+    w_k[q] = (lpos ^ R) * 8;
+#pragma unroll
+    for (int j = 0; j < CT; ++j) {
+      // the row within the workgroup's columns, and where it lies from the descriptor's base
+      const int col = GLU ? wave * 16 + R : wave * CT * 16 + 16 * j + R;
+      const unsigned row = static_cast<unsigned>(col) + ((GLU && j == 1) ? static_cast<unsigned>(N) : 0u);
+      w_at[j][q] = (wg_row0 + col < N) ? row * static_cast<unsigned>(ldw) * 2u + 2u * w_k[q] : GR_OOB;
+    }
+  }
+  // Operand reads: lane (r, g) takes piece 4 s + g of row r of a tile.
+  unsigned piece_at[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) piece_at[s] = (r >> 2) * 1024 + (r & 3) * 256 + (((4 * s + g) ^ r) * 16);
+
   floatx4 acc[CT][MT];
 #pragma unroll
   for (int j = 0; j < CT; ++j)
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[j][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  // The loads of chunk C into stage S.  A chunk beyond the range issues the same loads with
+  // The loads of chunk c into a stage.  A chunk beyond the range issues the same loads with
   // every offset out of range: nothing is fetched, and the count of loads per turn stays fixed.
-#define GR_ISSUE(C, S)                                                                               \
-  do {                                                                                               \
-    const int k0 = (C) * GR_CHUNK;                                                                   \
-    const bool live = (C) < c_end;                                                                   \
-    _Pragma("unroll") for (int i = 0; i < XL; ++i) {                                                 \
-      const int k = k0 + x_step[i];                                                                  \
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(xres, (GR_LDS(void)*)(&xs[S][wave + GR_WAVES * i][0]),    \
-                                           16, (live && k < K) ? x_row[i] + 2u * k : GR_OOB, 0, 0, 0); \
-    }                                                                                                \
-    _Pragma("unroll") for (int j = 0; j < CT; ++j) _Pragma("unroll") for (int s = 0; s < 4; ++s) {   \
-      const int k = k0 + s * 32 + g * 8;                                                             \
-      const unsigned at = (live && k < K && w_row[j] != GR_OOB) ? w_row[j] + 2u * k : GR_OOB;        \
-      wreg[S][j][s] = __builtin_amdgcn_raw_buffer_load_b128(wres, at, 0, 0);                                \
-    }                                                                                                \
-  } while (0)
+  auto issue = [&](int c, int stage) {
+    const bool live = c < c_end;
+    const unsigned k0 = static_cast<unsigned>(c) * GR_CHUNK;
+    unsigned char* base = lds + stage * Shape::STAGE_BYTES;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const bool ok = live && x_at[t] != GR_OOB && static_cast<int>(k0) + x_k < K;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(xres, (GR_LDS(void)*)(base + t * GR_TILE_BYTES + wave * 1024), 16,
+                                               ok ? x_at[t] + 2u * k0 : GR_OOB, 0, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < CT; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const bool ok = live && w_at[j][q] != GR_OOB && static_cast<int>(k0) + w_k[q] < K;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            wres, (GR_LDS(void)*)(base + (MT + wave * CT + j) * GR_TILE_BYTES + q * 1024), 16,
+            ok ? w_at[j][q] + 2u * k0 : GR_OOB, 0, 0, 0);
+      }
+  };
+  auto compute = [&](int stage) {
+    const GR_LDS(unsigned char)* base = (const GR_LDS(unsigned char)*)(lds + stage * Shape::STAGE_BYTES);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      bf16x8 xf[MT], wf[CT];
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        xf[t] = *reinterpret_cast<const GR_LDS(bf16x8)*>(base + t * GR_TILE_BYTES + piece_at[s]);
+#pragma unroll
+      for (int j = 0; j < CT; ++j)
+        wf[j] = *reinterpret_cast<const GR_LDS(bf16x8)*>(base + (MT + wave * CT + j) * GR_TILE_BYTES + piece_at[s]);
+#pragma unroll
+      for (int j = 0; j < CT; ++j)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], xf[t], acc[j][t], 0, 0, 0);
+    }
+  };
 
-#define GR_COMPUTE(S)                                                                                \
-  do {                                                                                               \
-    _Pragma("unroll") for (int s = 0; s < 4; ++s) {                                                  \
-      bf16x8 xf[MT];                                                                                 \
-      _Pragma("unroll") for (int t = 0; t < MT; ++t)                                                 \
-        xf[t] = *reinterpret_cast<const GR_LDS(bf16x8)*>(                                            \
-            (const GR_LDS(unsigned char)*)(&xs[S][4 * t + s][0]) + lane * 16);                       \
-      _Pragma("unroll") for (int j = 0; j < CT; ++j) _Pragma("unroll") for (int t = 0; t < MT; ++t)  \
-        acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(                                         \
-            __builtin_bit_cast(bf16x8, wreg[S][j][s]), xf[t], acc[j][t], 0, 0, 0);                   \
-    }                                                                                                \
-  } while (0)
-
-  // Chunk c lives in stage c % 3.  On entry the loads of chunks c and c + 1 are outstanding;
-  // chunk c has landed once at most those of c + 1 are.  After the barrier every wave is past
-  // the products of chunk c - 1, whose stage chunk c + 2 takes.
-#define GR_TURN(S)                                                                                   \
-  do {                                                                                               \
-    __builtin_amdgcn_sched_barrier(0); /* the counted wait relies on the order of issue */          \
-    gr_wait_loads<LOADS>();                                                                          \
-    gr_barrier();                                                                                    \
-    __builtin_amdgcn_sched_barrier(0);                                                               \
-    GR_ISSUE(c + 2, ((S) + 2) % GR_STAGES);                                                          \
-    __builtin_amdgcn_sched_barrier(0);                                                               \
-    GR_COMPUTE(S);                                                                                   \
-    ++c;                                                                                             \
-  } while (0)
-
-  // Turns come in threes without a way out in between: a branch after a turn would let the
-  // compiler sink that turn's loads of w behind it, next to their first use.  Up to two turns
-  // past the range multiply zeros.
-  int c = c_begin;
-  GR_ISSUE(c, 0);
-  __builtin_amdgcn_sched_barrier(0);
-  GR_ISSUE(c + 1, 1);
-  for (int rounds = (c_end - c_begin + GR_STAGES - 1) / GR_STAGES; rounds > 0; --rounds) {
-    GR_TURN(0);
-    GR_TURN(1);
-    GR_TURN(2);
+  // Chunk c lives in stage (c - c_begin) % STAGES.  At the top of turn c the loads of chunks
+  // c .. c + STAGES - 2 are outstanding; chunk c has landed once at most those of the later
+  // ones are.  After the barrier every wave is past the products of chunk c - 1, whose stage
+  // chunk c + STAGES - 1 takes.
+#pragma unroll
+  for (int i = 0; i < STAGES - 1; ++i) issue(c_begin + i, i);
+  int stage = 0;
+  for (int c = c_begin; c < c_end; ++c) {
+    gr_wait_loads<LOADS*(STAGES - 2)>();
+    gr_barrier();
+    issue(c + STAGES - 1, stage == 0 ? STAGES - 1 : stage - 1);
+    compute(stage);
+    stage = (stage + 1 == STAGES) ? 0 : stage + 1;
   }
-#undef GR_TURN
-#undef GR_COMPUTE
-#undef GR_ISSUE
 
-  // acc[j][t][i] is out[16 t + r][n0 + 16 j + 4 g + i]
+  // acc[j][t][i] is out[16 t + r][n0 + 16 j + 4 g + i] (with GLU: gate and up of column
+  // n0 + 4 g + i).  Four values of a lane go out as one store where every row of every part
+  // is aligned for it.
   TO* dst = out + static_cast<size_t>(part) * part_stride;
-  // four sums of a lane go out as one 16-byte store where every row of every part is aligned
-  const bool wide = sizeof(TO) == 4 && (ldo & 3) == 0 && (part_stride & 3) == 0 &&
-                    (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+  const bool wide = (ldo & 3) == 0 && (part_stride & 3) == 0 &&
+                    (reinterpret_cast<uintptr_t>(out) & (4 * sizeof(TO) - 1)) == 0;
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = t * 16 + r;
     if (m >= M) continue;
 #pragma unroll
-    for (int j = 0; j < CT; ++j) {
+    for (int j = 0; j < (GLU ? 1 : CT); ++j) {
       const int n = n0 + 16 * j + 4 * g;
-      TO* p = dst + static_cast<size_t>(m) * ldo + n;
-      if constexpr (sizeof(TO) == 4) {
-        if (wide && n + 3 < N) {
-          *reinterpret_cast<floatx4*>(p) = acc[j][t];
-          continue;
-        }
-      }
+      floatx4 v = acc[j][t];
+      if constexpr (GLU) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (n + i < N) p[i] = from_float<TO>(acc[j][t][i]);
+        for (int i = 0; i < 4; ++i) v[i] = gr_silu(acc[0][t][i]) * acc[1][t][i];
+      }
+      TO* p = dst + static_cast<size_t>(m) * ldo + n;
+      if (wide && n + 3 < N) {
+        if constexpr (sizeof(TO) == 4) {
+          *reinterpret_cast<floatx4*>(p) = v;
+        } else {
+          uint2 packed;
+          packed.x = float_to_bf16_bits(v[0]) | (static_cast<uint32_t>(float_to_bf16_bits(v[1])) << 16);
+          packed.y = float_to_bf16_bits(v[2]) | (static_cast<uint32_t>(float_to_bf16_bits(v[3])) << 16);
+          *reinterpret_cast<uint2*>(p) = packed;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < N) p[i] = from_float<TO>(v[i]);
+      }
     }
   }
 }
 
-template <int MT, int CT, typename TO>
+template <int MT, int CT, bool GLU, typename TO>
 __global__ __launch_bounds__(GR_WAVES* PYLON_WAVE) void gemm_rows_kernel(
     TO* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int M, int N,
     int K, long long ldx, long long ldw, long long ldo, long long part_stride, int chunks_per_part) {
-  gemm_rows_body<MT, CT, TO>(out, x, w, M, N, K, ldx, ldw, ldo, part_stride, chunks_per_part);
+  gemm_rows_body<MT, CT, GLU, TO>(out, x, w, M, N, K, ldx, ldw, ldo, part_stride, chunks_per_part);
 }
 
-template <int MT, int CT>
+template <int MT, int CT, bool GLU>
 static void launch_rows(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                         long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
                         hipStream_t stream) {
   const int chunks = (K + GR_CHUNK - 1) / GR_CHUNK;
   const int per_part = (chunks + parts - 1) / parts;
-  dim3 grid((N + GR_WAVES * CT * 16 - 1) / (GR_WAVES * CT * 16), parts), block(GR_WAVES * PYLON_WAVE);
+  constexpr int WG_COLS = GR_WAVES * (GLU ? 1 : CT) * 16;
+  dim3 grid((N + WG_COLS - 1) / WG_COLS, parts), block(GR_WAVES * PYLON_WAVE);
   if (out_dtype == PYLON_F32)
-    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, float>), grid, block, 0, stream, (float*)out,
+    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, GLU, float>), grid, block, 0, stream, (float*)out,
                        (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part);
   else
-    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, bf16_t>), grid, block, 0, stream, (bf16_t*)out,
+    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, GLU, bf16_t>), grid, block, 0, stream, (bf16_t*)out,
                        (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part);
 }
 
-// x: [M, ldx] bf16, 1 <= M <= 64; w: [N, ldw] bf16; out: `parts` results [M, ldo] spaced
-// part_stride elements apart (parts > 1 needs float out).  col_tiles: tiles of 16 columns per
-// wave, 1 or 2 (a workgroup then covers 64 or 128 columns).
+// x: [M, ldx] bf16, 1 <= M <= 64; w: [N, ldw] bf16 (with glu: [2N, ldw], gate rows first, then
+// up rows); out: `parts` results [M, ldo] spaced part_stride elements apart (parts > 1 needs
+// float out and no glu).  col_tiles: tiles of 16 columns per wave, 1 or 2 (a workgroup then
+// covers 64 or 128 columns); with glu a wave takes 16 gate rows and their 16 up rows, and a
+// workgroup covers 64 columns.
 extern "C" int pylon_gemm_rows(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                                long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
-                               int col_tiles, hipStream_t stream) {
+                               int col_tiles, int glu, hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(out_dtype), "gemm_rows: unknown output dtype");
   PYLON_REQUIRE(M >= 0 && M <= 64, "gemm_rows: takes at most 64 rows, got %d", M);
   PYLON_REQUIRE(N > 0 && K > 0, "gemm_rows: bad sizes N=%d K=%d", N, K);
@@ -227,13 +268,18 @@ extern "C" int pylon_gemm_rows(void* out, int out_dtype, const void* x, const vo
   PYLON_REQUIRE(col_tiles == 1 || col_tiles == 2, "gemm_rows: col_tiles is 1 or 2, got %d", col_tiles);
   PYLON_REQUIRE(parts >= 1 && parts <= 64, "gemm_rows: parts must be 1..64");
   PYLON_REQUIRE(parts == 1 || out_dtype == PYLON_F32, "gemm_rows: partial results must be float");
+  PYLON_REQUIRE(parts == 1 || !glu, "gemm_rows: the gated epilogue needs the whole of K");
   PYLON_REQUIRE(parts == 1 || part_stride >= static_cast<long long>(M) * ldo,
                 "gemm_rows: partial results overlap");
+  PYLON_REQUIRE(!glu || (static_cast<long long>(N) + 64) * ldw * 2 < (1ll << 31),
+                "gemm_rows: a fused gate/up matrix of %d rows of %lld elements is beyond the 2 GB a "
+                "workgroup's view of it may span", 2 * N, ldw);
   if (M == 0) return 0;
 #define GO(MT)                                                                                              \
   do {                                                                                                      \
-    if (col_tiles == 2) launch_rows<MT, 2>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream); \
-    else launch_rows<MT, 1>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream);      \
+    if (glu) launch_rows<MT, 2, true>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream); \
+    else if (col_tiles == 2) launch_rows<MT, 2, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream); \
+    else launch_rows<MT, 1, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream); \
   } while (0)
   switch ((M + 15) / 16) {
     case 1: GO(1); break;

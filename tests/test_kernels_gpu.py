@@ -249,6 +249,16 @@ def test_gemm_rows(ops, shape):
     assert torch.equal(alone[:, 0], full[:, m // 2])
     with pytest.raises(Exception, match="at most 64 rows"):
         ops.gemm_rows(rnd((65, k), 34, torch.bfloat16).to(DEV), w.to(DEV))
+    # gated epilogue over a fused gate/up matrix equals the product, then the activation
+    if n % 2 == 0:
+        g, u = want[:, : n // 2], want[:, n // 2:]
+        want_glu = g / (1 + np.exp(-g)) * u
+        for out_dtype in (torch.bfloat16, torch.float32):
+            fused = ops.gemm_rows(a.to(DEV), w.to(DEV), out_dtype=out_dtype, glu=True)
+            assert fused.shape == (m, n // 2) and fused.dtype == out_dtype
+            assert np.abs(f64(fused) - want_glu).max() <= tol(out_dtype, np.abs(want_glu).max())
+        with pytest.raises(Exception, match="whole of K"):
+            ops.gemm_rows(a.to(DEV), w.to(DEV), parts=2, glu=True)
 
 
 def test_rows_plan_keeps_the_workgroups_within_the_chip(ops):
