@@ -31,7 +31,6 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 #define GR_CHUNK 128
 #define GR_TILE_BYTES 4096  // 16 rows of one chunk
-#define GR_WAVES 4
 #define GR_LDS(T) __attribute__((address_space(3))) T
 #define GR_OOB 0x80000000u
 
@@ -49,10 +48,10 @@ __device__ __forceinline__ void gr_wait_loads() {
   __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
 }
 
-// Stages of LDS for MT tiles of x and 4 * CT tiles of w per chunk: as many as fit, at most 4.
-template <int MT, int CT>
+// Stages of LDS for MT tiles of x and WAVES * CT tiles of w per chunk: as many as fit, at most 4.
+template <int MT, int CT, int WAVES>
 struct GrShape {
-  static constexpr int TILES = MT + GR_WAVES * CT;
+  static constexpr int TILES = MT + WAVES * CT;
   static constexpr int STAGE_BYTES = TILES * GR_TILE_BYTES;
   static constexpr int STAGES = (4 * STAGE_BYTES <= 144 * 1024) ? 4 : 3;
 };
@@ -62,21 +61,22 @@ struct GrShape {
 // its second the 16 up rows that lie N rows further down, and it writes silu(gate) * up.
 // (The body is a device function: the host pass does not know the descriptor type and would
 // drop a kernel that names it, launch stub and all.)
-template <int MT, int CT, bool GLU, typename TO>
+template <int MT, int CT, bool GLU, int WAVES, typename TO>
 __device__ __forceinline__ void gemm_rows_body(
     TO* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int M, int N,
     int K, long long ldx, long long ldw, long long ldo, long long part_stride, int chunks_per_part) {
-  typedef GrShape<MT, CT> Shape;
+  typedef GrShape<MT, CT, WAVES> Shape;
+  constexpr int QW = 4 / WAVES;  // quarters of every tile of x that a wave fills
   constexpr int STAGES = Shape::STAGES;
-  constexpr int LOADS = MT + 4 * CT;  // loads a wave issues per chunk
+  constexpr int LOADS = QW * MT + 4 * CT;  // loads a wave issues per chunk
   __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * Shape::STAGE_BYTES];
 
   const int lane = threadIdx.x & (PYLON_WAVE - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PYLON_WAVE);
   const int r = lane & 15, g = lane >> 4;
-  constexpr int WG_COLS = GR_WAVES * (GLU ? 1 : CT) * 16;  // columns of the output per workgroup
+  constexpr int WG_COLS = WAVES * (GLU ? 1 : CT) * 16;  // columns of the output per workgroup
   const int wg_row0 = blockIdx.x * WG_COLS;                // first row of w of this workgroup
-  const int n0 = wg_row0 + wave * (WG_COLS / GR_WAVES);    // and of this wave
+  const int n0 = wg_row0 + wave * (WG_COLS / WAVES);       // and of this wave
   const int part = blockIdx.y;
   const int chunks = (K + GR_CHUNK - 1) / GR_CHUNK;
   const int c_begin = part * chunks_per_part;
@@ -93,18 +93,19 @@ __device__ __forceinline__ void gemm_rows_body(
 
   // A load fills rows 4 q .. 4 q + 3 of a tile (q: the quarter): lane l brings, for row
   // R = 4 q + l / 16, the piece (l % 16) ^ R.
-  // x: this wave fills quarter `wave` of every tile of x.
+  // x: this wave fills quarters QW * wave .. of every tile of x.
   const int lrow = lane >> 4, lpos = lane & 15;
-  unsigned x_at[MT];  // byte offset of this lane's piece in chunk 0, or out of range
-  int x_k;            // its first element within a chunk
-  {
-    const int R = 4 * wave + lrow;
-    x_k = (lpos ^ R) * 8;
+  unsigned x_at[QW][MT];  // byte offset of this lane's piece in chunk 0, or out of range
+  int x_k[QW];            // its first element within a chunk
+#pragma unroll
+  for (int u = 0; u < QW; ++u) {
+    const int R = 4 * (QW * wave + u) + lrow;
+    x_k[u] = (lpos ^ R) * 8;
 #pragma unroll
     for (int t = 0; t < MT; ++t)
-      x_at[t] = (16 * t + R < M)
-                    ? static_cast<unsigned>(16 * t + R) * static_cast<unsigned>(ldx) * 2u + 2u * x_k
-                    : GR_OOB;
+      x_at[u][t] = (16 * t + R < M)
+                       ? static_cast<unsigned>(16 * t + R) * static_cast<unsigned>(ldx) * 2u + 2u * x_k[u]
+                       : GR_OOB;
   }
   // w: this wave fills all four quarters of its own CT tiles.
   unsigned w_at[CT][4];
@@ -139,11 +140,14 @@ __device__ __forceinline__ void gemm_rows_body(
     const unsigned k0 = static_cast<unsigned>(c) * GR_CHUNK;
     unsigned char* base = lds + stage * Shape::STAGE_BYTES;
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const bool ok = live && x_at[t] != GR_OOB && static_cast<int>(k0) + x_k < K;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(xres, (GR_LDS(void)*)(base + t * GR_TILE_BYTES + wave * 1024), 16,
-                                               ok ? x_at[t] + 2u * k0 : GR_OOB, 0, 0, 0);
-    }
+    for (int u = 0; u < QW; ++u)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const bool ok = live && x_at[u][t] != GR_OOB && static_cast<int>(k0) + x_k[u] < K;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            xres, (GR_LDS(void)*)(base + t * GR_TILE_BYTES + (QW * wave + u) * 1024), 16,
+            ok ? x_at[u][t] + 2u * k0 : GR_OOB, 0, 0, 0);
+      }
 #pragma unroll
     for (int j = 0; j < CT; ++j)
 #pragma unroll
@@ -225,37 +229,48 @@ __device__ __forceinline__ void gemm_rows_body(
   }
 }
 
-template <int MT, int CT, bool GLU, typename TO>
-__global__ __launch_bounds__(GR_WAVES* PYLON_WAVE) void gemm_rows_kernel(
+template <int MT, int CT, bool GLU, int WAVES, typename TO>
+__global__ __launch_bounds__(WAVES* PYLON_WAVE) void gemm_rows_kernel(
     TO* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int M, int N,
     int K, long long ldx, long long ldw, long long ldo, long long part_stride, int chunks_per_part) {
-  gemm_rows_body<MT, CT, GLU, TO>(out, x, w, M, N, K, ldx, ldw, ldo, part_stride, chunks_per_part);
+  gemm_rows_body<MT, CT, GLU, WAVES, TO>(out, x, w, M, N, K, ldx, ldw, ldo, part_stride, chunks_per_part);
 }
 
+template <int MT, int CT, bool GLU, int WAVES>
+static void launch_rows_waves(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
+                              long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
+                              hipStream_t stream) {
+  const int chunks = (K + GR_CHUNK - 1) / GR_CHUNK;
+  const int per_part = (chunks + parts - 1) / parts;
+  constexpr int WG_COLS = WAVES * (GLU ? 1 : CT) * 16;
+  dim3 grid((N + WG_COLS - 1) / WG_COLS, parts), block(WAVES * PYLON_WAVE);
+  if (out_dtype == PYLON_F32)
+    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, GLU, WAVES, float>), grid, block, 0, stream, (float*)out,
+                       (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part);
+  else
+    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, GLU, WAVES, bf16_t>), grid, block, 0, stream, (bf16_t*)out,
+                       (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part);
+}
+
+// Workgroups of four waves, or of two where four would leave compute units without one.
 template <int MT, int CT, bool GLU>
 static void launch_rows(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                         long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
-                        hipStream_t stream) {
-  const int chunks = (K + GR_CHUNK - 1) / GR_CHUNK;
-  const int per_part = (chunks + parts - 1) / parts;
-  constexpr int WG_COLS = GR_WAVES * (GLU ? 1 : CT) * 16;
-  dim3 grid((N + WG_COLS - 1) / WG_COLS, parts), block(GR_WAVES * PYLON_WAVE);
-  if (out_dtype == PYLON_F32)
-    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, GLU, float>), grid, block, 0, stream, (float*)out,
-                       (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part);
+                        int waves, hipStream_t stream) {
+  if (waves == 2)
+    launch_rows_waves<MT, CT, GLU, 2>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream);
   else
-    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, GLU, bf16_t>), grid, block, 0, stream, (bf16_t*)out,
-                       (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part);
+    launch_rows_waves<MT, CT, GLU, 4>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream);
 }
 
 // x: [M, ldx] bf16, 1 <= M <= 64; w: [N, ldw] bf16 (with glu: [2N, ldw], gate rows first, then
 // up rows); out: `parts` results [M, ldo] spaced part_stride elements apart (parts > 1 needs
-// float out and no glu).  col_tiles: tiles of 16 columns per wave, 1 or 2 (a workgroup then
-// covers 64 or 128 columns); with glu a wave takes 16 gate rows and their 16 up rows, and a
-// workgroup covers 64 columns.
+// float out and no glu).  col_tiles: tiles of 16 columns per wave, 1 or 2; with glu a wave
+// takes 16 gate rows and their 16 up rows.  waves: wavefronts per workgroup, 4 or 2 (0: two if
+// four would give fewer than 128 workgroups).
 extern "C" int pylon_gemm_rows(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                                long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
-                               int col_tiles, int glu, hipStream_t stream) {
+                               int col_tiles, int glu, int waves, hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(out_dtype), "gemm_rows: unknown output dtype");
   PYLON_REQUIRE(M >= 0 && M <= 64, "gemm_rows: takes at most 64 rows, got %d", M);
   PYLON_REQUIRE(N > 0 && K > 0, "gemm_rows: bad sizes N=%d K=%d", N, K);
@@ -274,12 +289,17 @@ extern "C" int pylon_gemm_rows(void* out, int out_dtype, const void* x, const vo
   PYLON_REQUIRE(!glu || (static_cast<long long>(N) + 64) * ldw * 2 < (1ll << 31),
                 "gemm_rows: a fused gate/up matrix of %d rows of %lld elements is beyond the 2 GB a "
                 "workgroup's view of it may span", 2 * N, ldw);
+  PYLON_REQUIRE(waves == 0 || waves == 2 || waves == 4, "gemm_rows: waves is 0, 2 or 4, got %d", waves);
   if (M == 0) return 0;
+  if (waves == 0) {
+    const int cols = 4 * 16 * (glu ? 1 : col_tiles);
+    waves = (static_cast<long long>((N + cols - 1) / cols) * parts < 128) ? 2 : 4;
+  }
 #define GO(MT)                                                                                              \
   do {                                                                                                      \
-    if (glu) launch_rows<MT, 2, true>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream); \
-    else if (col_tiles == 2) launch_rows<MT, 2, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream); \
-    else launch_rows<MT, 1, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream); \
+    if (glu) launch_rows<MT, 2, true>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, waves, stream); \
+    else if (col_tiles == 2) launch_rows<MT, 2, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, waves, stream); \
+    else launch_rows<MT, 1, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, waves, stream); \
   } while (0)
   switch ((M + 15) / 16) {
     case 1: GO(1); break;

@@ -487,14 +487,15 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype
 
 
 def gemm_rows(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype = torch.bfloat16,
-              parts: int = 1, col_tiles: int = 1, glu: bool = False,
+              parts: int = 1, col_tiles: int = 1, glu: bool = False, waves: int = 0,
               out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ weight.T`` for at most 64 rows of bfloat16 ``x``, made for 17 to 64: the rows of
     ``x`` pass through LDS once per workgroup of 64 (``col_tiles=1``) or 128 (``col_tiles=2``)
     columns and ``weight`` is streamed once.  ``parts > 1`` cuts K into that many ranges and
     returns float32 partial results ``[parts, M, N]`` for the consumer to add.  ``glu``:
     ``weight`` is a fused ``[2N, K]`` gate/up matrix and the result is
-    ``silu(x @ gate.T) * (x @ up.T)``, rounded once."""
+    ``silu(x @ gate.T) * (x @ up.T)``, rounded once.  ``waves``: wavefronts per workgroup,
+    4 or 2 (0: the kernel's choice); the sums do not depend on it."""
     if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
         raise KernelError(f"gemm_rows: cannot multiply {tuple(x.shape)} by the transpose of {tuple(weight.shape)}")
     m, k = x.shape
@@ -514,7 +515,8 @@ def gemm_rows(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype =
             or not out.is_cuda or not out.is_contiguous():
         raise KernelError(f"gemm_rows: out must be contiguous, on the GPU and of shape {shape}")
     _lib.call("pylon_gemm_rows", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), weight.data_ptr(),
-              m, n, k, x.stride(0), weight.stride(0), n, parts, m * n, int(col_tiles), 1 if glu else 0, _stream())
+              m, n, k, x.stride(0), weight.stride(0), n, parts, m * n, int(col_tiles), 1 if glu else 0, int(waves),
+              _stream())
     return out
 
 
@@ -545,11 +547,11 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.d
            out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ weight.T`` (into ``out`` if given: contiguous, of the result's shape and type).
 
-    bfloat16 by bfloat16: up to 16 rows go to the weight-streaming kernel, more rows to the
-    library matrix product (as the reference's ``nn.Linear`` does).  With a bfloat16 result
-    the float32 sums are rounded once either way; with a float32 result (the logits) they
-    come back unrounded either way (the library then writes its float32 sums): what a
-    request's logits are rounded to does not depend on how many rows share its step.
+    bfloat16 by bfloat16: up to 64 rows go to a weight-streaming kernel where one is faster,
+    more rows to the library matrix product (as the reference's ``nn.Linear`` does).  With a
+    bfloat16 result the float32 sums are rounded once either way; with a float32 result (the
+    logits) they come back unrounded either way (the library then writes its float32 sums):
+    what a request's logits are rounded to does not depend on how many rows share its step.
     Every pairing that involves float32 operands runs on the exact tiled kernel, which never
     uses a reduced-precision matrix mode.
     """
@@ -557,13 +559,23 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.d
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
         if not x.is_cuda:
             raise KernelError("linear: operands must live on the GPU; there is no CPU path")
-        if skinny_ok(x, weight):
-            return gemm_skinny(x, weight, out_dtype=out_dtype, out=out)
+        n, k = weight.shape
+        few = skinny_ok(x, weight)
+        if n >= TALL_ROWS:
+            # a vocabulary head: up to 16 rows the kernel whose waves split K (152 us for a
+            # 151936 x 2560 matrix); 17 to 64 rows the one that shares x through LDS (172
+            # against the library's 190 us at 64 rows, 149 against 174 at 24)
+            if few:
+                return gemm_skinny(x, weight, out_dtype=out_dtype, out=out)
+            if _streaming_ok(x, weight, STREAM_ROWS):
+                return gemm_rows(x, weight, out_dtype=out_dtype, col_tiles=2, out=out)
+        elif few or (_streaming_ok(x, weight, STREAM_ROWS) and k % 4096):
+            # a projection: measured at 8 rows 6144 x 2560 9.3 against 10.7 us of the kernel
+            # whose waves split K, 10240 x 5120 21 against 31; at 48 rows 13.6 against the
+            # library's 15.5 and 29 against 32.  Rows of a power-of-two length beyond 16 rows
+            # stay with the library (6144 x 4096 at 48 rows: 19 against 18).
+            return gemm_rows(x, weight, out_dtype=out_dtype, out=out)
         if out_dtype == torch.float32:
-            if weight.shape[0] >= TALL_ROWS and _streaming_ok(x, weight, STREAM_ROWS) and x.is_contiguous():
-                # a vocabulary head for 17 to 64 rows: measured 172 against the library's 190 us
-                # at 64 rows of a 151936 x 2560 matrix, 149 against 174 at 24
-                return gemm_rows(x, weight, out_dtype=torch.float32, col_tiles=2, out=out)
             return _library_float(x, weight, out)
         y = torch.nn.functional.linear(x, weight)
         y = y if out_dtype == torch.bfloat16 else y.to(out_dtype)
@@ -578,13 +590,14 @@ def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: tor
     for 17 to 64 rows of a matrix at which the library is faster, the library's float32
     result.  For more rows (prompt portions) it is the library's product rounded once to
     bfloat16."""
-    if skinny_ok(x, weight):
-        return gemm_skinny(x, weight, out_dtype=out_dtype, parts=k_parts(*weight.shape))
     if _streaming_ok(x, weight, STREAM_ROWS):
         n, k = weight.shape
-        if deep_or_small(n, k):
-            parts, col_tiles = rows_plan(n, k)
+        few = x.shape[0] <= SKINNY_ROWS
+        if deep_or_small(n, k) or (few and n <= 8192):
+            parts, col_tiles = rows_plan(n, k, x.shape[0])
             return gemm_rows(x, weight, out_dtype=torch.float32, parts=parts, col_tiles=col_tiles)
+        if few:
+            return gemm_skinny(x, weight, out_dtype=out_dtype, parts=k_parts(n, k))
         return _library_float(x, weight)
     return linear(x, weight, out_dtype=out_dtype)
 
@@ -593,18 +606,21 @@ def deep_or_small(n: int, k: int) -> bool:
     """Shapes at which, for 17 to 64 rows, the kernel that shares the rows of x through LDS
     and cuts K into parts beats the library product: matrices much deeper than wide (a down
     projection; the library does not cut K) and those of few rows (an out projection).
-    Measured at 64 rows: 2560x4096 11 against 14 us, 2560x9728 21 against 28, 4096x4096 12
-    against 15, 4096x12288 29 against 39, 5120x25600 79 against 90; but 5120x8192 30 against
-    29 and 8192x8192 39 against 35, which stay with the library."""
+    Measured at 64 rows: 2560x4096 9.5 against 14 us, 2560x9728 17 against 28, 4096x4096 11
+    against 15, 4096x12288 24 against 39, 5120x25600 79 against 90; but 5120x8192 30 against
+    29 and 8192x8192 39 against 35, which stay with the library.  (Up to 16 rows the same
+    kernel also beats the one whose waves split K: 2560x4096 6.2 against 8.3 us at 8 rows,
+    2560x9728 11.5 against 13.8, 5120x8192 20 against 23, 5120x25600 52 against 65.)"""
     return k >= 2 * n or n <= 4096
 
 
-def rows_plan(n: int, k: int) -> tuple:
+def rows_plan(n: int, k: int, rows: int = STREAM_ROWS) -> tuple:
     """(parts, col_tiles) for :func:`gemm_rows` on an ``[n, k]`` matrix: workgroups of 128
-    columns for deep matrices, else of 64, and K cut into the largest power of two of parts
-    (at most 16, of at least 256 elements each) that keeps the workgroups at 256 or fewer, one
-    per compute unit: more of them only re-read the rows of x."""
-    col_tiles = 2 if k >= 8192 else 1
+    columns for deep matrices (beyond 16 rows, where the rows of x weigh more, from a depth
+    of 8192) and for wide ones, else of 64; K cut into the largest power of two of parts (at
+    most 16, of at least 256 elements each) that keeps the workgroups at 256 or fewer, one per
+    compute unit: more of them only re-read the rows of x."""
+    col_tiles = 2 if (k >= 8192 and rows > SKINNY_ROWS) or k >= 16384 or n > 4096 else 1
     groups = -(-n // (64 * col_tiles))
     parts = 1
     while parts < 16 and 2 * parts * groups <= 256 and k // (2 * parts) >= 256:
@@ -615,17 +631,21 @@ def rows_plan(n: int, k: int) -> tuple:
 def linear_glu(x: torch.Tensor, gate_up: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:
     """``silu(x @ gate.T) * (x @ up.T)`` for a fused ``[2I, K]`` gate/up matrix.  Up to 64
     bfloat16 rows: the activation works on the float32 sums and its result is rounded once
-    (in a streaming kernel's epilogue; beyond 16 rows of a matrix wider than 4096, where that
-    kernel no longer beats the library, from the library's float32 result).  More rows
-    (prompt portions): the library's product rounded to bfloat16 first."""
-    if skinny_ok(x, gate_up):
-        return gemm_skinny(x, gate_up, out_dtype=out_dtype, glu=True)
-    if _streaming_ok(x, gate_up, STREAM_ROWS) and x.is_cuda:
+    (in a streaming kernel's epilogue; or, where the library is faster, from its float32
+    result).  More rows (prompt portions): the library's product rounded to bfloat16 first."""
+    if _streaming_ok(x, gate_up, STREAM_ROWS) and x.is_cuda and gate_up.shape[0] % 2 == 0:
         two_i, k = gate_up.shape
-        # measured at 64 rows: 2x9728 x 2560 27 against 34 us, 2x12288 x 4096 48 against 55,
-        # 2x25600 x 5120 113 against 113
-        if k <= 4096 and two_i % 2 == 0 and (two_i // 2 + 64) * gate_up.stride(0) * 2 < 2 ** 31:
+        few = x.shape[0] <= SKINNY_ROWS
+        fits = (two_i // 2 + 64) * gate_up.stride(0) * 2 < 2 ** 31  # a workgroup's view of gate and up rows
+        # The kernel that shares x through LDS, measured against the one whose waves split K
+        # at 8 rows: 2x9728 x 2560 22 against 25 us, 2x25600 x 5120 98 against 109, 2x6144 x 2048
+        # 12 against 15; but 2x12288 x 4096 44 against 40 (rows of a power-of-two length of 8 KB
+        # or more) and 2x3072 x 1024 6.7 against 6.1.  Against the library and the activation
+        # kernel at 64 rows: 27 against 34 us, 48 against 55 (width 4096), 113 against 113 (5120).
+        if fits and (k <= 4096 if not few else (k % 4096 != 0 and two_i >= 8192)):
             return gemm_rows(x, gate_up, out_dtype=out_dtype, glu=True)
+        if few:
+            return gemm_skinny(x, gate_up, out_dtype=out_dtype, glu=True)
         return silu_gate(_library_float(x, gate_up), out_dtype=out_dtype)
     return silu_gate(linear(x, gate_up, out_dtype=out_dtype))
 
