@@ -64,7 +64,8 @@ struct GrShape {
 template <int MT, int CT, bool GLU, int WAVES, typename TO>
 __device__ __forceinline__ void gemm_rows_body(
     TO* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int M, int N,
-    int K, long long ldx, long long ldw, long long ldo, long long part_stride, int chunks_per_part) {
+    int K, long long ldx, long long ldw, long long ldo, long long part_stride, int chunks_per_part,
+    int spread) {
   typedef GrShape<MT, CT, WAVES> Shape;
   constexpr int QW = 4 / WAVES;  // quarters of every tile of x that a wave fills
   constexpr int STAGES = Shape::STAGES;
@@ -74,17 +75,22 @@ __device__ __forceinline__ void gemm_rows_body(
   const int lane = threadIdx.x & (PYLON_WAVE - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PYLON_WAVE);
   const int r = lane & 15, g = lane >> 4;
-  constexpr int WG_COLS = WAVES * (GLU ? 1 : CT) * 16;  // columns of the output per workgroup
-  const int wg_row0 = blockIdx.x * WG_COLS;                // first row of w of this workgroup
-  const int n0 = wg_row0 + wave * (WG_COLS / WAVES);       // and of this wave
+  constexpr int WAVE_COLS = (GLU ? 1 : CT) * 16;  // columns of the output per wave
+  constexpr int WG_COLS = WAVES * WAVE_COLS;
+  // A workgroup's waves take neighbouring groups of columns, or, spread, groups that lie
+  // gridDim.x apart: a matrix of 608 groups then keeps 256 workgroups (two or three waves
+  // of each) busy instead of 152.
+  const int wg_row0 = spread ? 0 : blockIdx.x * WG_COLS;  // first row of w the descriptor covers
+  const int n0 = spread ? (blockIdx.x + gridDim.x * wave) * WAVE_COLS : wg_row0 + wave * WAVE_COLS;
   const int part = blockIdx.y;
   const int chunks = (K + GR_CHUNK - 1) / GR_CHUNK;
   const int c_begin = part * chunks_per_part;
   const int c_end = (c_begin + chunks_per_part < chunks) ? c_begin + chunks_per_part : chunks;
 
   // The descriptor of w starts at the workgroup's first row (with GLU it reaches N rows
-  // further, to its up rows: the host checks that this fits 31 bits).
-  const int wg_rows = (N - wg_row0 < WG_COLS) ? N - wg_row0 : WG_COLS;
+  // further, to its up rows; spread, it covers the matrix: the host checks that this fits
+  // 31 bits).
+  const int wg_rows = (spread || N - wg_row0 < WG_COLS) ? N - wg_row0 : WG_COLS;
   const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t*>(w + static_cast<size_t>(wg_row0) * ldw), 0,
       static_cast<int>((static_cast<long long>((GLU ? N : 0) + wg_rows - 1) * ldw + K) * 2), 0x00020000);
@@ -117,7 +123,7 @@ __device__ __forceinline__ void gemm_rows_body(
 #pragma unroll
     for (int j = 0; j < CT; ++j) {
       // the row within the workgroup's columns, and where it lies from the descriptor's base
-      const int col = GLU ? wave * 16 + R : wave * CT * 16 + 16 * j + R;
+      const int col = n0 - wg_row0 + (GLU ? R : 16 * j + R);
       const unsigned row = static_cast<unsigned>(col) + ((GLU && j == 1) ? static_cast<unsigned>(N) : 0u);
       w_at[j][q] = (wg_row0 + col < N) ? row * static_cast<unsigned>(ldw) * 2u + 2u * w_k[q] : GR_OOB;
     }
@@ -232,8 +238,9 @@ __device__ __forceinline__ void gemm_rows_body(
 template <int MT, int CT, bool GLU, int WAVES, typename TO>
 __global__ __launch_bounds__(WAVES* PYLON_WAVE) void gemm_rows_kernel(
     TO* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int M, int N,
-    int K, long long ldx, long long ldw, long long ldo, long long part_stride, int chunks_per_part) {
-  gemm_rows_body<MT, CT, GLU, WAVES, TO>(out, x, w, M, N, K, ldx, ldw, ldo, part_stride, chunks_per_part);
+    int K, long long ldx, long long ldw, long long ldo, long long part_stride, int chunks_per_part,
+    int spread) {
+  gemm_rows_body<MT, CT, GLU, WAVES, TO>(out, x, w, M, N, K, ldx, ldw, ldo, part_stride, chunks_per_part, spread);
 }
 
 template <int MT, int CT, bool GLU, int WAVES>
@@ -242,14 +249,23 @@ static void launch_rows_waves(void* out, int out_dtype, const void* x, const voi
                               hipStream_t stream) {
   const int chunks = (K + GR_CHUNK - 1) / GR_CHUNK;
   const int per_part = (chunks + parts - 1) / parts;
-  constexpr int WG_COLS = WAVES * (GLU ? 1 : CT) * 16;
-  dim3 grid((N + WG_COLS - 1) / WG_COLS, parts), block(WAVES * PYLON_WAVE);
+  constexpr int WAVE_COLS = (GLU ? 1 : CT) * 16;
+  const int tasks = (N + WAVE_COLS - 1) / WAVE_COLS;  // groups of columns, one per wave
+  int groups = (tasks + WAVES - 1) / WAVES;
+  // Between 256 and 256 * WAVES groups of a matrix that one descriptor can cover: 256
+  // workgroups whose waves take groups 256 apart, so that every compute unit has one.
+  const int spread = parts == 1 && tasks > 256 && groups < 256 &&
+                     static_cast<long long>(GLU ? 2 * N : N) * ldw * 2 < (1ll << 31);
+  if (spread) groups = 256;
+  dim3 grid(groups, parts), block(WAVES * PYLON_WAVE);
   if (out_dtype == PYLON_F32)
     hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, GLU, WAVES, float>), grid, block, 0, stream, (float*)out,
-                       (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part);
+                       (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part,
+                       spread);
   else
     hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, GLU, WAVES, bf16_t>), grid, block, 0, stream, (bf16_t*)out,
-                       (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part);
+                       (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part,
+                       spread);
 }
 
 // Workgroups of four waves, or of two where four would leave compute units without one.
