@@ -293,7 +293,8 @@ extern "C" int pylon_gemm_rows(void* out, int out_dtype, const void* x, const vo
   PYLON_REQUIRE(K % 8 == 0, "gemm_rows: K=%d must be a multiple of 8", K);
   PYLON_REQUIRE(ldx % 8 == 0 && ldw % 8 == 0, "gemm_rows: row strides must be multiples of 8 elements");
   PYLON_REQUIRE(ldw >= K && ldx >= K && ldo >= N, "gemm_rows: a row stride is too short");
-  PYLON_REQUIRE(ldw <= (1ll << 22), "gemm_rows: rows of w longer than 4M elements are not supported");
+  PYLON_REQUIRE(ldw <= (1ll << 22) && ldx <= (1ll << 22),
+                "gemm_rows: row strides beyond 4M elements are not supported");
   PYLON_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0,
                 "gemm_rows: operands must be 16-byte aligned");
   PYLON_REQUIRE(col_tiles == 1 || col_tiles == 2, "gemm_rows: col_tiles is 1 or 2, got %d", col_tiles);

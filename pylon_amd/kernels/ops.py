@@ -562,10 +562,11 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.d
         n, k = weight.shape
         few = skinny_ok(x, weight)
         if n >= TALL_ROWS:
-            # a vocabulary head: up to 16 rows the kernel whose waves split K (152 us for a
-            # 151936 x 2560 matrix); 17 to 64 rows the one that shares x through LDS (172
-            # against the library's 190 us at 64 rows, 149 against 174 at 24)
-            if few:
+            # a vocabulary head: the kernel that shares x through LDS (151936 x 2560 at 8 rows:
+            # 136 us against 154 of the kernel whose waves split K; at 64 rows 172 against the
+            # library's 190, at 24 rows 149 against 174), except up to 16 rows of a
+            # power-of-two length of 8 KB (x 4096: 239 against 237)
+            if few and k % 4096 == 0:
                 return gemm_skinny(x, weight, out_dtype=out_dtype, out=out)
             if _streaming_ok(x, weight, STREAM_ROWS):
                 return gemm_rows(x, weight, out_dtype=out_dtype, col_tiles=2, out=out)

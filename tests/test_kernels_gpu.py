@@ -245,6 +245,12 @@ def test_gemm_rows(ops, shape):
     assert torch.equal(alone[:, 0], full[:, m // 2])
     with pytest.raises(Exception, match="at most 64 rows"):
         ops.gemm_rows(rnd((65, k), 34, torch.bfloat16).to(DEV), w.to(DEV))
+    # rows of x and w that are slices of wider tensors (strides beyond K)
+    wide_x = rnd((m, k + 24), 35, torch.bfloat16).to(DEV)
+    wide_w = rnd((n, k + 40), 36, torch.bfloat16, 0.1).to(DEV)
+    sliced = ops.gemm_rows(wide_x[:, 8: 8 + k], wide_w[:, 16: 16 + k], out_dtype=torch.float32)
+    want_sliced = f64(wide_x[:, 8: 8 + k]) @ f64(wide_w[:, 16: 16 + k]).T
+    assert np.abs(f64(sliced) - want_sliced).max() <= tol(torch.float32, np.abs(want_sliced).max())
     # gated epilogue over a fused gate/up matrix equals the product, then the activation
     if n % 2 == 0:
         g, u = want[:, : n // 2], want[:, n // 2:]
