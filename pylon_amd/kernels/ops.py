@@ -10,6 +10,7 @@ from typing import Optional
 import torch
 
 from . import library as _lib
+from . import plan
 from .library import KernelError
 
 F32 = 0
@@ -433,25 +434,16 @@ def gemm_tiled(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[tor
     return out
 
 
-# Most rows of x for which the first weight-streaming kernel is chosen.  It takes up to 64,
-# but beyond one 16-row tile it re-reads x once per 16 weight rows, and the library's tiled
-# kernels measured faster (e.g. 27 us against 64 us for the fused gate/up matrix at 64 rows).
-# A variant that stages x in LDS and shares it between four waves was tried for 17..64 rows:
-# it stayed behind the library too (43 us for that matrix), and where cutting K over
-# workgroups put it ahead (12 us against 19 us for a 2560 x 4096 matrix) the residual norm
-# paid the gain back by adding eight partial results of 64 rows.
-SKINNY_ROWS = 16
+SKINNY_ROWS = plan.FEW_ROWS    # one tile of rows of x
+STREAM_ROWS = plan.STREAM_ROWS  # most rows of x one launch of a weight-streaming kernel takes
 
 
 def _streaming_ok(x: torch.Tensor, weight: torch.Tensor, rows: int) -> bool:
+    """Operands a weight-streaming kernel takes: bfloat16, at most ``rows`` rows of x, rows of
+    multiples of 8 elements at 16-byte aligned addresses."""
     return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < x.shape[0] <= rows
             and weight.shape[1] % 8 == 0 and weight.stride(0) % 8 == 0 and x.stride(0) % 8 == 0
             and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
-
-
-def skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Few rows: the kernel whose waves split K and read x straight from memory."""
-    return _streaming_ok(x, weight, SKINNY_ROWS)
 
 
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype = torch.bfloat16,
@@ -520,21 +512,6 @@ def gemm_rows(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype =
     return out
 
 
-def k_parts(n: int, k: int) -> int:
-    """How many ranges to cut K into so that a matrix with few rows still fills the chip.
-    At most 4: with 8 (and two-tile workgroups, the best pairing for the products alone) a
-    whole decode step measured 7 % slower."""
-    tiles = (n + 15) // 16
-    parts = 1
-    while tiles * parts < 512 and parts < 4 and k // (parts * 2) >= 512:
-        parts *= 2
-    return parts
-
-
-STREAM_ROWS = 64  # most rows of x one launch of a weight-streaming kernel takes
-TALL_ROWS = 32768  # a matrix of at least this many rows (a vocabulary head) is "tall"
-
-
 def _library_float(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ weight.T`` of bfloat16 operands as float32: the library's product with a float32
     result, that is its float32 sums before any rounding."""
@@ -547,35 +524,24 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.d
            out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ weight.T`` (into ``out`` if given: contiguous, of the result's shape and type).
 
-    bfloat16 by bfloat16: up to 64 rows go to a weight-streaming kernel where one is faster,
-    more rows to the library matrix product (as the reference's ``nn.Linear`` does).  With a
-    bfloat16 result the float32 sums are rounded once either way; with a float32 result (the
-    logits) they come back unrounded either way (the library then writes its float32 sums):
-    what a request's logits are rounded to does not depend on how many rows share its step.
-    Every pairing that involves float32 operands runs on the exact tiled kernel, which never
-    uses a reduced-precision matrix mode.
+    bfloat16 by bfloat16: up to 64 rows go to a weight-streaming kernel where one is faster
+    (:func:`plan.plan_projection`), more rows to the library matrix product (as the
+    reference's ``nn.Linear`` does).  With a bfloat16 result the float32 sums are rounded once
+    either way; with a float32 result (the logits) they come back unrounded either way (the
+    library then writes its float32 sums): what a request's logits are rounded to does not
+    depend on how many rows share its step.  Every pairing that involves float32 operands runs
+    on the exact tiled kernel, which never uses a reduced-precision matrix mode.
     """
     out_dtype = out_dtype or x.dtype
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
         if not x.is_cuda:
             raise KernelError("linear: operands must live on the GPU; there is no CPU path")
-        n, k = weight.shape
-        few = skinny_ok(x, weight)
-        if n >= TALL_ROWS:
-            # a vocabulary head: the kernel that shares x through LDS (151936 x 2560 at 8 rows:
-            # 136 us against 154 of the kernel whose waves split K; at 64 rows 172 against the
-            # library's 190, at 24 rows 149 against 174), except up to 16 rows of a
-            # power-of-two length of 8 KB (x 4096: 239 against 237)
-            if few and k % 4096 == 0:
+        if _streaming_ok(x, weight, STREAM_ROWS):
+            choice = plan.plan_projection(x.shape[0], *weight.shape)
+            if choice.kernel == "rows":
+                return gemm_rows(x, weight, out_dtype=out_dtype, col_tiles=choice.col_tiles, out=out)
+            if choice.kernel == "skinny":
                 return gemm_skinny(x, weight, out_dtype=out_dtype, out=out)
-            if _streaming_ok(x, weight, STREAM_ROWS):
-                return gemm_rows(x, weight, out_dtype=out_dtype, col_tiles=2, out=out)
-        elif few or (_streaming_ok(x, weight, STREAM_ROWS) and k % 4096):
-            # a projection: measured at 8 rows 6144 x 2560 9.3 against 10.7 us of the kernel
-            # whose waves split K, 10240 x 5120 21 against 31; at 48 rows 13.6 against the
-            # library's 15.5 and 29 against 32.  Rows of a power-of-two length beyond 16 rows
-            # stay with the library (6144 x 4096 at 48 rows: 19 against 18).
-            return gemm_rows(x, weight, out_dtype=out_dtype, out=out)
         if out_dtype == torch.float32:
             return _library_float(x, weight, out)
         y = torch.nn.functional.linear(x, weight)
@@ -589,63 +555,29 @@ def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: tor
     to 64 bfloat16 rows it comes back as unrounded float32 sums, which the fused residual norm
     adds: partial sums ``[parts, M, N]`` of a streaming kernel (K cut over workgroups), or,
     for 17 to 64 rows of a matrix at which the library is faster, the library's float32
-    result.  For more rows (prompt portions) it is the library's product rounded once to
-    bfloat16."""
+    result (:func:`plan.plan_residual`).  For more rows (prompt portions) it is the library's
+    product rounded once to bfloat16."""
     if _streaming_ok(x, weight, STREAM_ROWS):
-        n, k = weight.shape
-        few = x.shape[0] <= SKINNY_ROWS
-        if deep_or_small(n, k) or (few and n <= 8192):
-            parts, col_tiles = rows_plan(n, k, x.shape[0])
-            return gemm_rows(x, weight, out_dtype=torch.float32, parts=parts, col_tiles=col_tiles)
-        if few:
-            return gemm_skinny(x, weight, out_dtype=out_dtype, parts=k_parts(n, k))
+        choice = plan.plan_residual(x.shape[0], *weight.shape)
+        if choice.kernel == "rows":
+            return gemm_rows(x, weight, out_dtype=torch.float32, parts=choice.parts, col_tiles=choice.col_tiles)
+        if choice.kernel == "skinny":
+            return gemm_skinny(x, weight, out_dtype=torch.float32, parts=choice.parts)
         return _library_float(x, weight)
     return linear(x, weight, out_dtype=out_dtype)
-
-
-def deep_or_small(n: int, k: int) -> bool:
-    """Shapes at which, for 17 to 64 rows, the kernel that shares the rows of x through LDS
-    and cuts K into parts beats the library product: matrices much deeper than wide (a down
-    projection; the library does not cut K) and those of few rows (an out projection).
-    Measured at 64 rows: 2560x4096 9.5 against 14 us, 2560x9728 17 against 28, 4096x4096 11
-    against 15, 4096x12288 24 against 39, 5120x25600 79 against 90; but 5120x8192 30 against
-    29 and 8192x8192 39 against 35, which stay with the library.  (Up to 16 rows the same
-    kernel also beats the one whose waves split K: 2560x4096 6.2 against 8.3 us at 8 rows,
-    2560x9728 11.5 against 13.8, 5120x8192 20 against 23, 5120x25600 52 against 65.)"""
-    return k >= 2 * n or n <= 4096
-
-
-def rows_plan(n: int, k: int, rows: int = STREAM_ROWS) -> tuple:
-    """(parts, col_tiles) for :func:`gemm_rows` on an ``[n, k]`` matrix: workgroups of 128
-    columns for deep matrices (beyond 16 rows, where the rows of x weigh more, from a depth
-    of 8192) and for wide ones, else of 64; K cut into the largest power of two of parts (at
-    most 16, of at least 256 elements each) that keeps the workgroups at 256 or fewer, one per
-    compute unit: more of them only re-read the rows of x."""
-    col_tiles = 2 if (k >= 8192 and rows > SKINNY_ROWS) or k >= 16384 or n > 4096 else 1
-    groups = -(-n // (64 * col_tiles))
-    parts = 1
-    while parts < 16 and 2 * parts * groups <= 256 and k // (2 * parts) >= 256:
-        parts *= 2
-    return parts, col_tiles
 
 
 def linear_glu(x: torch.Tensor, gate_up: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:
     """``silu(x @ gate.T) * (x @ up.T)`` for a fused ``[2I, K]`` gate/up matrix.  Up to 64
     bfloat16 rows: the activation works on the float32 sums and its result is rounded once
     (in a streaming kernel's epilogue; or, where the library is faster, from its float32
-    result).  More rows (prompt portions): the library's product rounded to bfloat16 first."""
+    result: :func:`plan.plan_gated`).  More rows (prompt portions): the library's product
+    rounded to bfloat16 first."""
     if _streaming_ok(x, gate_up, STREAM_ROWS) and x.is_cuda and gate_up.shape[0] % 2 == 0:
-        two_i, k = gate_up.shape
-        few = x.shape[0] <= SKINNY_ROWS
-        fits = (two_i // 2 + 64) * gate_up.stride(0) * 2 < 2 ** 31  # a workgroup's view of gate and up rows
-        # The kernel that shares x through LDS, measured against the one whose waves split K
-        # at 8 rows: 2x9728 x 2560 22 against 25 us, 2x25600 x 5120 98 against 109, 2x6144 x 2048
-        # 12 against 15; but 2x12288 x 4096 44 against 40 (rows of a power-of-two length of 8 KB
-        # or more) and 2x3072 x 1024 6.7 against 6.1.  Against the library and the activation
-        # kernel at 64 rows: 27 against 34 us, 48 against 55 (width 4096), 113 against 113 (5120).
-        if fits and (k <= 4096 if not few else (k % 4096 != 0 and two_i >= 8192)):
+        choice = plan.plan_gated(x.shape[0], gate_up.shape[0] // 2, gate_up.shape[1], gate_up.stride(0))
+        if choice.kernel == "rows":
             return gemm_rows(x, gate_up, out_dtype=out_dtype, glu=True)
-        if few:
+        if choice.kernel == "skinny":
             return gemm_skinny(x, gate_up, out_dtype=out_dtype, glu=True)
         return silu_gate(_library_float(x, gate_up), out_dtype=out_dtype)
     return silu_gate(linear(x, gate_up, out_dtype=out_dtype))

@@ -1,0 +1,119 @@
+"""Which kernel multiplies a few rows of bfloat16 activations by a bfloat16 matrix.
+
+Pure functions of the shape: they touch no tensor and run anywhere, so the choices can be
+tested without a GPU.  Every figure below was measured on one MI355X, under a graph, over 36
+different matrices in turn (so that none came from a cache).
+
+Three kernels take part.  ``rows`` (``gemm_rows``): both operands go through LDS in whole
+256-byte row segments, the rows of x are shared by a workgroup, K may be cut over workgroups.
+``skinny`` (``gemm_skinny``): the earlier one, whose waves split K and read x in the shape of
+a matrix-instruction operand.  ``library``: the library's tiled product.  Up to 64 rows the
+product is bound by moving the matrix once, and by what a compute unit can pull: the first
+kernel wins almost everywhere; the exceptions are listed where they are decided.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+FEW_ROWS = 16      # one tile of rows of x
+STREAM_ROWS = 64   # most rows of x a weight-streaming kernel takes
+TALL = 32768       # a matrix of at least this many rows (a vocabulary head) is "tall"
+UNITS = 256        # compute units
+
+
+@dataclass(frozen=True)
+class Product:
+    """``kernel``: "rows", "skinny" or "library"; ``parts``: ranges K is cut into (each a float
+    partial result for the consumer to add); ``col_tiles``: tiles of 16 columns per wave of
+    the rows kernel."""
+    kernel: str
+    parts: int = 1
+    col_tiles: int = 1
+
+
+def aliased_rows(k: int) -> bool:
+    """Rows of a power-of-two length of 8 KB or more: the 256-byte segments that a chunk is of
+    many rows then meet in few memory channels, and the rows kernel streams 10 to 20 % slower
+    (gate/up 2x12288 x 4096 at 8 rows: 44 us against the skinny kernel's 40)."""
+    return k % 4096 == 0
+
+
+def rows_split(n: int, k: int, rows: int = STREAM_ROWS) -> tuple:
+    """(parts, col_tiles) of the rows kernel for a product into the residual stream.
+    Workgroups of 128 columns for deep matrices (beyond 16 rows, where the rows of x weigh
+    more, from a depth of 8192) and for wide ones, else of 64; K cut into the largest power of
+    two of parts (at most 16, of at least 256 elements each) that keeps the workgroups at 256
+    or fewer, one per compute unit: more of them only re-read the rows of x."""
+    col_tiles = 2 if (k >= 8192 and rows > FEW_ROWS) or k >= 16384 or n > 4096 else 1
+    groups = -(-n // (64 * col_tiles))
+    parts = 1
+    while parts < 16 and 2 * parts * groups <= UNITS and k // (2 * parts) >= 256:
+        parts *= 2
+    return parts, col_tiles
+
+
+def skinny_parts(n: int, k: int) -> int:
+    """Ranges the skinny kernel cuts K into so that a matrix of few rows still fills the chip
+    (at most 4: with 8 a whole decode step measured 7 % slower)."""
+    tiles = (n + 15) // 16
+    parts = 1
+    while tiles * parts < 512 and parts < 4 and k // (parts * 2) >= 512:
+        parts *= 2
+    return parts
+
+
+def deep_or_narrow(n: int, k: int) -> bool:
+    """Matrices much deeper than wide (a down projection; the library does not cut K) and
+    those of few rows (an out projection): there the rows kernel with K cut into parts beats
+    the library at 17 to 64 rows.  At 64 rows: 2560x4096 9.5 against 14 us, 2560x9728 17
+    against 28, 4096x4096 11 against 15, 4096x12288 24 against 39, 5120x25600 79 against 90;
+    but 5120x8192 30 against 29 and 8192x8192 39 against 35."""
+    return k >= 2 * n or n <= 4096
+
+
+def plan_residual(rows: int, n: int, k: int) -> Product:
+    """A product about to be added to the float32 residual stream (out and down projections),
+    ``rows`` <= 64: float32 sums, never rounded, from whichever kernel.  Up to 16 rows the rows
+    kernel also beats the skinny one (2560x4096 at 8 rows: 6.2 against 8.3 us, 2560x9728 11.5
+    against 13.8, 5120x8192 20 against 23, 5120x25600 52 against 65)."""
+    few = rows <= FEW_ROWS
+    if deep_or_narrow(n, k) or (few and n <= 8192):
+        parts, col_tiles = rows_split(n, k, rows)
+        return Product("rows", parts, col_tiles)
+    if few:
+        return Product("skinny", skinny_parts(n, k))
+    return Product("library")
+
+
+def plan_projection(rows: int, n: int, k: int) -> Product:
+    """Any other product of ``rows`` <= 64 (q/k/v; the vocabulary head).
+
+    A head (tall matrix): the rows kernel with 128 columns per workgroup (151936 x 2560: 136 us
+    against the skinny kernel's 154 at 8 rows; 172 against the library's 190 at 64 rows, 149
+    against 174 at 24), except up to 16 rows of aliased rows (x 4096: 239 against 237).
+    A projection: the rows kernel (6144 x 2560 at 8 rows 9.3 against 10.7 us, 10240 x 5120 21
+    against 31; at 48 rows 13.6 against the library's 15.5 and 29 against 32), except beyond 16
+    rows of aliased rows (6144 x 4096 at 48 rows: 19 against the library's 18)."""
+    few = rows <= FEW_ROWS
+    if n >= TALL:
+        return Product("skinny") if few and aliased_rows(k) else Product("rows", 1, 2)
+    if few or not aliased_rows(k):
+        return Product("rows")
+    return Product("library")
+
+
+def plan_gated(rows: int, n_half: int, k: int, row_stride: int) -> Product:
+    """``silu(x gate^T) * (x up^T)`` over a fused matrix of ``2 * n_half`` rows, ``rows`` <= 64;
+    "library" means its float32 result followed by the activation kernel.
+
+    Against the skinny kernel at 8 rows: 2x9728 x 2560 21 against 25 us, 2x25600 x 5120 98
+    against 109, 2x6144 x 2048 12 against 15; but 2x12288 x 4096 44 against 40 (aliased rows)
+    and 2x3072 x 1024 6.7 against 6.1 (a small matrix).  Against the library and the
+    activation kernel at 64 rows: 27 against 34 us, 48 against 55 (width 4096), 113 against
+    113 (width 5120).  A workgroup of the rows kernel sees its gate rows and, ``n_half`` rows
+    further, its up rows through one descriptor, which spans at most 2 GB."""
+    few = rows <= FEW_ROWS
+    fits = (n_half + 64) * row_stride * 2 < 2 ** 31
+    if fits and ((not aliased_rows(k) and n_half >= 4096) if few else k <= 4096):
+        return Product("rows", 1, 2)
+    return Product("skinny") if few else Product("library")

@@ -263,14 +263,6 @@ def test_gemm_rows(ops, shape):
             ops.gemm_rows(a.to(DEV), w.to(DEV), parts=2, glu=True)
 
 
-def test_rows_plan_keeps_the_workgroups_within_the_chip(ops):
-    for n, k in [(2560, 4096), (2560, 9728), (4096, 12288), (5120, 25600), (1024, 2048), (64, 512), (100, 256)]:
-        parts, col_tiles = ops.rows_plan(n, k)
-        groups = -(-n // (64 * col_tiles))
-        assert col_tiles in (1, 2) and 1 <= parts <= 16
-        assert parts == 1 or (parts * groups <= 256 and k // parts >= 256)
-
-
 def plain_rope(x, pos, inv_freq, rot):
     # x: [..., d]; rotate the first `rot` elements, pairing i with i + rot/2
     ang = (np.float32(pos) * inv_freq.astype(np.float32)).astype(np.float64)

@@ -1,0 +1,78 @@
+"""The choice of product kernel by shape (pylon_amd/kernels/plan.py): pure functions, checked
+here without a GPU for the sizes of every Qwen3 dense model and for the properties the
+kernels rely on."""
+import pytest
+
+from pylon_amd.kernels import plan
+
+# (hidden, q width, key/value width, feed-forward width) of the published Qwen3 dense sizes
+SIZES = {
+    "0.6b": (1024, 2048, 1024, 3072),
+    "1.7b": (2048, 2048, 1024, 6144),
+    "4b": (2560, 4096, 1024, 9728),
+    "8b": (4096, 4096, 1024, 12288),
+    "14b": (5120, 5120, 1024, 17408),
+    "32b": (5120, 8192, 1024, 25600),
+}
+VOCAB = 151936
+
+
+@pytest.mark.parametrize("rows", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("name", list(SIZES))
+def test_every_choice_is_one_the_kernels_take(name, rows):
+    hidden, q, kv, inter = SIZES[name]
+    for n, k in ((hidden, q), (hidden, inter)):
+        c = plan.plan_residual(rows, n, k)
+        assert c.kernel in ("rows", "skinny", "library")
+        if c.kernel == "rows":
+            groups = -(-n // (64 * c.col_tiles))
+            assert c.col_tiles in (1, 2) and 1 <= c.parts <= 16
+            assert c.parts == 1 or (c.parts * groups <= plan.UNITS and k // c.parts >= 256)
+        if c.kernel == "skinny":
+            assert rows <= plan.FEW_ROWS and 1 <= c.parts <= 4
+    for n, k in ((q + 2 * kv, hidden), (VOCAB, hidden)):
+        c = plan.plan_projection(rows, n, k)
+        assert c.parts == 1  # nothing adds partial sums behind these
+        assert c.kernel != "skinny" or rows <= plan.FEW_ROWS
+    c = plan.plan_gated(rows, inter, hidden, hidden)
+    assert c.parts == 1 and (c.kernel != "skinny" or rows <= plan.FEW_ROWS)
+    assert c.kernel != "rows" or c.col_tiles == 2  # a wave's gate tile and its up tile
+
+
+def test_the_benchmark_shape_streams_everything_through_the_rows_kernel():
+    hidden, q, kv, inter = SIZES["4b"]
+    for rows in (1, 8, 16, 64):
+        assert plan.plan_projection(rows, q + 2 * kv, hidden).kernel == "rows"
+        assert plan.plan_projection(rows, VOCAB, hidden) == plan.Product("rows", 1, 2)
+        assert plan.plan_gated(rows, inter, hidden, hidden).kernel == "rows"
+        assert plan.plan_residual(rows, hidden, q) == plan.Product("rows", 4, 1)
+    assert plan.plan_residual(8, hidden, inter) == plan.Product("rows", 4, 1)
+    assert plan.plan_residual(64, hidden, inter) == plan.Product("rows", 8, 2)
+
+
+def test_rows_of_a_power_of_two_length_and_small_matrices_keep_the_other_kernels():
+    hidden, q, kv, inter = SIZES["8b"]
+    assert plan.aliased_rows(hidden) and not plan.aliased_rows(2560) and not plan.aliased_rows(2048)
+    assert plan.plan_gated(8, inter, hidden, hidden).kernel == "skinny"
+    assert plan.plan_gated(64, inter, hidden, hidden).kernel == "rows"
+    assert plan.plan_projection(48, q + 2 * kv, hidden).kernel == "library"
+    assert plan.plan_projection(8, q + 2 * kv, hidden).kernel == "rows"
+    assert plan.plan_projection(8, VOCAB, hidden).kernel == "skinny"
+    assert plan.plan_gated(8, 3072, 1024, 1024).kernel == "skinny"      # a small matrix
+    assert plan.plan_gated(64, 25600, 5120, 5120).kernel == "library"   # wider than 4096
+    assert plan.plan_residual(64, 8192, 8192).kernel == "library"       # wide and shallow
+    assert plan.plan_residual(8, 16384, 8192).kernel == "skinny"
+
+
+def test_a_gate_up_matrix_beyond_a_descriptor_is_not_given_to_the_rows_kernel():
+    assert plan.plan_gated(8, 300_000, 2560, 4096).kernel == "skinny"   # 300,064 rows x 8 KB > 2 GB
+    assert plan.plan_gated(64, 300_000, 2560, 4096).kernel == "library"
+
+
+def test_parts_are_powers_of_two_and_independent_of_the_row_count_within_a_class():
+    for n, k in [(2560, 4096), (2560, 9728), (4096, 12288), (5120, 25600), (1024, 2048), (64, 512), (100, 256)]:
+        few = {plan.rows_split(n, k, rows) for rows in (1, 8, 16)}
+        many = {plan.rows_split(n, k, rows) for rows in (17, 33, 64)}
+        assert len(few) == 1 and len(many) == 1  # one order of additions per class of row counts
+        for parts, col_tiles in few | many:
+            assert parts & (parts - 1) == 0 and col_tiles in (1, 2)
