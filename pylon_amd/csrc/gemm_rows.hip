@@ -197,6 +197,9 @@ __device__ __forceinline__ void gemm_rows_body(
     compute(stage);
     stage = (stage + 1 == STAGES) ? 0 : stage + 1;
   }
+  // The loads still outstanding are those past the range: they fetch nothing but do write
+  // (zeros) into LDS when they complete, so the wave sees them through before it leaves.
+  gr_wait_loads<0>();
 
   // acc[j][t][i] is out[16 t + r][n0 + 16 j + 4 g + i] (with GLU: gate and up of column
   // n0 + 4 g + i).  Four values of a lane go out as one store where every row of every part
