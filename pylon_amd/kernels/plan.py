@@ -91,15 +91,16 @@ def plan_projection(rows: int, n: int, k: int) -> Product:
     A head (tall matrix): the rows kernel with 128 columns per workgroup (151936 x 2560: 136 us
     against the skinny kernel's 154 at 8 rows; 172 against the library's 190 at 64 rows, 149
     against 174 at 24), except up to 16 rows of aliased rows (x 4096: 239 against 237).
-    A projection: the rows kernel (6144 x 2560 at 8 rows 9.3 against 10.7 us, 10240 x 5120 21
-    against 31; at 48 rows 13.6 against the library's 15.5 and 29 against 32), except beyond 16
-    rows of aliased rows (6144 x 4096 at 48 rows: 19 against the library's 18)."""
+    A projection up to 16 rows: the rows kernel (6144 x 2560 at 8 rows 9.3 against the skinny
+    kernel's 10.7 us, 10240 x 5120 21 against 31, 6144 x 4096 13.5 against 16).  Beyond 16
+    rows the library: the rows kernel is within 10 % of it either way (6144 x 2560: 14.4
+    against 15.4 us at 48 rows, 17.2 against 15.5 at 64; 7168 x 5120: 24 against 23 and 30
+    against 24; 10240 x 5120: 28 against 32 and 31 against 33), and the rows of x of a
+    workgroup that covers 64 of many columns weigh most here."""
     few = rows <= FEW_ROWS
     if n >= TALL:
         return Product("skinny") if few and aliased_rows(k) else Product("rows", 1, 2)
-    if few or not aliased_rows(k):
-        return Product("rows")
-    return Product("library")
+    return Product("rows") if few else Product("library")
 
 
 def plan_gated(rows: int, n_half: int, k: int, row_stride: int) -> Product:

@@ -39,10 +39,10 @@ def test_every_choice_is_one_the_kernels_take(name, rows):
     assert c.kernel != "rows" or c.col_tiles == 2  # a wave's gate tile and its up tile
 
 
-def test_the_benchmark_shape_streams_everything_through_the_rows_kernel():
+def test_the_benchmark_shape_streams_nearly_everything_through_the_rows_kernel():
     hidden, q, kv, inter = SIZES["4b"]
     for rows in (1, 8, 16, 64):
-        assert plan.plan_projection(rows, q + 2 * kv, hidden).kernel == "rows"
+        assert plan.plan_projection(rows, q + 2 * kv, hidden).kernel == ("rows" if rows <= 16 else "library")
         assert plan.plan_projection(rows, VOCAB, hidden) == plan.Product("rows", 1, 2)
         assert plan.plan_gated(rows, inter, hidden, hidden).kernel == "rows"
         assert plan.plan_residual(rows, hidden, q) == plan.Product("rows", 4, 1)
