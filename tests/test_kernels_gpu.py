@@ -217,6 +217,31 @@ def test_gemm_skinny(ops, shape):
         ops.gemm_skinny(torch.zeros((65, 64), dtype=torch.bfloat16, device=DEV), w[:, :64].contiguous().to(DEV))
 
 
+def test_gemm_rows_at_random_shapes(ops):
+    """Sixty seeded draws of every argument (rows 1 to 64, 1 to 700 columns, depths that are
+    multiples of 8 up to 1,496, parts beyond the number of chunks, both widths and wave
+    counts, the gated form) against a float64 product."""
+    rng = np.random.default_rng(2024)
+    for case in range(60):
+        m = int(rng.integers(1, 65))
+        k = 8 * int(rng.integers(1, 188))
+        glu = bool(rng.integers(0, 2))
+        n = int(rng.integers(1, 351)) * (2 if glu else 1) if glu else int(rng.integers(1, 701))
+        parts = 1 if glu else int(rng.choice([1, 1, 2, 3, 5, 16]))
+        col_tiles, waves = int(rng.choice([1, 2])), int(rng.choice([0, 2, 4]))
+        a, w = rnd((m, k), 100 + case, torch.bfloat16), rnd((n, k), 200 + case, torch.bfloat16, 0.1)
+        want = f64(a) @ f64(w).T
+        if glu:
+            g, u = want[:, : n // 2], want[:, n // 2:]
+            want = g / (1 + np.exp(-g)) * u
+        got = ops.gemm_rows(a.to(DEV), w.to(DEV), out_dtype=torch.float32, parts=parts, col_tiles=col_tiles,
+                            glu=glu, waves=waves)
+        got = f64(got).sum(0) if parts > 1 else f64(got)
+        assert got.shape == want.shape, (case, m, n, k)
+        assert np.abs(got - want).max() <= tol(torch.float32, max(np.abs(want).max(), 1e-3)), \
+            (case, m, n, k, parts, col_tiles, glu, waves)
+
+
 @pytest.mark.parametrize("shape", [(17, 100, 200), (64, 2560 + 8, 512 + 24), (33, 61, 136), (50, 333, 1000),
                                    (64, 129, 128), (48, 64, 8), (20, 72, 9728), (1, 77, 264), (16, 300, 392)])
 def test_gemm_rows(ops, shape):
