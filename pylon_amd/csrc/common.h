@@ -111,5 +111,8 @@ extern thread_local char pylon_error_text[512];
     return 0;                                                                         \
   } while (0)
 
+// Compute units of the current device (0 if there is none); asked of the runtime once per device.
+extern "C" int pylon_compute_units();
+
 static inline bool pylon_valid_dtype(int d) { return d == PYLON_F32 || d == PYLON_BF16; }
 static inline size_t pylon_dtype_size(int d) { return d == PYLON_F32 ? 4 : 2; }

@@ -34,10 +34,13 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 #define GR_LDS(T) __attribute__((address_space(3))) T
 #define GR_OOB 0x80000000u
 
-// A bare barrier: the waits that must precede it are counted by hand below.  (A release
-// fence on LDS would wait for every outstanding load, because the loads that write LDS are
-// among them, and the chunks in flight would drain at every barrier.)
-__device__ __forceinline__ void gr_barrier() { asm volatile("s_barrier" ::: "memory"); }
+// A barrier behind a wait for this wave's reads of LDS only.  The invariant it keeps: when a
+// wave passes it, every wave's operand reads of the chunk before have returned, so the loads
+// issued next may overwrite that chunk's stage.  The loads from memory that must have landed
+// are counted by hand below and are not waited for here.  (A release fence on LDS would wait
+// for every outstanding load, because the loads that write LDS are among them, and the
+// chunks in flight would drain at every barrier.)
+__device__ __forceinline__ void gr_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 __device__ __forceinline__ float gr_silu(float z) { return z / (1.0f + expf(-z)); }
 
@@ -246,20 +249,35 @@ __global__ __launch_bounds__(WAVES* PYLON_WAVE) void gemm_rows_kernel(
   gemm_rows_body<MT, CT, GLU, WAVES, TO>(out, x, w, M, N, K, ldx, ldw, ldo, part_stride, chunks_per_part, spread);
 }
 
+// How a product is laid over the chip: wavefronts per workgroup, workgroups along the columns,
+// and whether a workgroup's waves take column groups that lie `groups` apart.
+struct GrLaunch {
+  int waves, groups, spread;
+};
+
+// units: compute units of the device.  waves: 4, 2, or 0 for two where four would give fewer
+// workgroups than half the units.
+static GrLaunch gr_launch_shape(int N, long long ldw, int parts, int col_tiles, int glu, int waves, int units) {
+  const int wave_cols = (glu ? 1 : col_tiles) * 16;
+  if (waves == 0)
+    waves = (static_cast<long long>((N + 4 * wave_cols - 1) / (4 * wave_cols)) * parts < units / 2) ? 2 : 4;
+  const int tasks = (N + wave_cols - 1) / wave_cols;  // groups of columns, one per wave
+  int groups = (tasks + waves - 1) / waves;
+  // Between `units` and `units * waves` groups of a matrix that one descriptor can cover: one
+  // workgroup per compute unit, whose waves take groups `units` apart.
+  const int spread = parts == 1 && tasks > units && groups < units &&
+                     static_cast<long long>(glu ? 2 * N : N) * ldw * 2 < (1ll << 31);
+  if (spread) groups = units;
+  return GrLaunch{waves, groups, spread};
+}
+
 template <int MT, int CT, bool GLU, int WAVES>
 static void launch_rows_waves(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                               long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
-                              hipStream_t stream) {
+                              const GrLaunch& shape, hipStream_t stream) {
   const int chunks = (K + GR_CHUNK - 1) / GR_CHUNK;
   const int per_part = (chunks + parts - 1) / parts;
-  constexpr int WAVE_COLS = (GLU ? 1 : CT) * 16;
-  const int tasks = (N + WAVE_COLS - 1) / WAVE_COLS;  // groups of columns, one per wave
-  int groups = (tasks + WAVES - 1) / WAVES;
-  // Between 256 and 256 * WAVES groups of a matrix that one descriptor can cover: 256
-  // workgroups whose waves take groups 256 apart, so that every compute unit has one.
-  const int spread = parts == 1 && tasks > 256 && groups < 256 &&
-                     static_cast<long long>(GLU ? 2 * N : N) * ldw * 2 < (1ll << 31);
-  if (spread) groups = 256;
+  const int groups = shape.groups, spread = shape.spread;
   dim3 grid(groups, parts), block(WAVES * PYLON_WAVE);
   if (out_dtype == PYLON_F32)
     hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, GLU, WAVES, float>), grid, block, 0, stream, (float*)out,
@@ -275,18 +293,34 @@ static void launch_rows_waves(void* out, int out_dtype, const void* x, const voi
 template <int MT, int CT, bool GLU>
 static void launch_rows(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                         long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
-                        int waves, hipStream_t stream) {
-  if (waves == 2)
-    launch_rows_waves<MT, CT, GLU, 2>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream);
+                        const GrLaunch& shape, hipStream_t stream) {
+  if (shape.waves == 2)
+    launch_rows_waves<MT, CT, GLU, 2>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, stream);
   else
-    launch_rows_waves<MT, CT, GLU, 4>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, stream);
+    launch_rows_waves<MT, CT, GLU, 4>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, stream);
+}
+
+// What pylon_gemm_rows would launch for these arguments on a device of `units` compute units
+// (0: the current device's): shape[0] wavefronts per workgroup, shape[1] workgroups along
+// the columns (times `parts` along K), shape[2] whether the waves' column groups are spread.
+// Touches no device memory; with units given it runs without a GPU.
+extern "C" int pylon_gemm_rows_shape(int N, long long ldw, int parts, int col_tiles, int glu, int waves,
+                                     int units, int* shape) {
+  PYLON_REQUIRE(shape != nullptr && N > 0 && parts >= 1, "gemm_rows_shape: bad arguments");
+  PYLON_REQUIRE(col_tiles == 1 || col_tiles == 2, "gemm_rows_shape: col_tiles is 1 or 2");
+  PYLON_REQUIRE(waves == 0 || waves == 2 || waves == 4, "gemm_rows_shape: waves is 0, 2 or 4");
+  if (units <= 0) units = pylon_compute_units();
+  PYLON_REQUIRE(units > 0, "gemm_rows_shape: no device to take the number of compute units from");
+  const GrLaunch l = gr_launch_shape(N, ldw, parts, col_tiles, glu, waves, units);
+  shape[0] = l.waves, shape[1] = l.groups, shape[2] = l.spread;
+  return 0;
 }
 
 // x: [M, ldx] bf16, 1 <= M <= 64; w: [N, ldw] bf16 (with glu: [2N, ldw], gate rows first, then
 // up rows); out: `parts` results [M, ldo] spaced part_stride elements apart (parts > 1 needs
 // float out and no glu).  col_tiles: tiles of 16 columns per wave, 1 or 2; with glu a wave
 // takes 16 gate rows and their 16 up rows.  waves: wavefronts per workgroup, 4 or 2 (0: two if
-// four would give fewer than 128 workgroups).
+// four would give fewer workgroups than half the device's compute units).
 extern "C" int pylon_gemm_rows(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                                long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
                                int col_tiles, int glu, int waves, hipStream_t stream) {
@@ -311,15 +345,14 @@ extern "C" int pylon_gemm_rows(void* out, int out_dtype, const void* x, const vo
                 "workgroup's view of it may span", 2 * N, ldw);
   PYLON_REQUIRE(waves == 0 || waves == 2 || waves == 4, "gemm_rows: waves is 0, 2 or 4, got %d", waves);
   if (M == 0) return 0;
-  if (waves == 0) {
-    const int cols = 4 * 16 * (glu ? 1 : col_tiles);
-    waves = (static_cast<long long>((N + cols - 1) / cols) * parts < 128) ? 2 : 4;
-  }
+  const int units = pylon_compute_units();
+  PYLON_REQUIRE(units > 0, "gemm_rows: the device's number of compute units is unknown");
+  const GrLaunch shape = gr_launch_shape(N, ldw, parts, col_tiles, glu, waves, units);
 #define GO(MT)                                                                                              \
   do {                                                                                                      \
-    if (glu) launch_rows<MT, 2, true>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, waves, stream); \
-    else if (col_tiles == 2) launch_rows<MT, 2, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, waves, stream); \
-    else launch_rows<MT, 1, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, waves, stream); \
+    if (glu) launch_rows<MT, 2, true>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, stream); \
+    else if (col_tiles == 2) launch_rows<MT, 2, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, stream); \
+    else launch_rows<MT, 1, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, stream); \
   } while (0)
   switch ((M + 15) / 16) {
     case 1: GO(1); break;

@@ -24,6 +24,25 @@ extern "C" int pylon_check_device() {
   return 0;
 }
 
+// Compute units of the current device, kept per device after the first question.
+extern "C" int pylon_compute_units() {
+  static int known[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  if (known[dev] == 0) {
+    int units = 0;
+    if (hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+      (void)hipGetLastError();
+      return 0;
+    }
+    known[dev] = units;
+  }
+  return known[dev];
+}
+
 // ---- a measurement aid: how fast can this device read memory? ---------------------------
 // Every thread reads 16 bytes at a time, eight loads in flight, and folds them into a word
 // nobody looks at (the store is never taken).  bench.py times it over a buffer larger than

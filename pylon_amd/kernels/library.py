@@ -38,6 +38,7 @@ _SIGNATURES = {
     "pylon_gemm_tiled": [P, I, P, I, P, I, I, I, I, L, L, L, P],
     "pylon_gemm_skinny": [P, I, P, P, I, I, I, L, L, L, I, L, I, P],
     "pylon_gemm_rows": [P, I, P, P, I, I, I, L, L, L, I, L, I, I, I, P],
+    "pylon_gemm_rows_shape": [I, L, I, I, I, I, I, P],
     "pylon_argmax": [P, P, I, I, L, P, P, P, L, P],
     "pylon_argmax_static": [P, P, I, I, L, P, P, P],
     "pylon_probe_read": [P, L, P, P],
@@ -50,6 +51,8 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.pylon_last_error.argtypes = []
     lib.pylon_abi_version.restype = c_int
     lib.pylon_check_device.restype = c_int
+    lib.pylon_compute_units.restype = c_int
+    lib.pylon_compute_units.argtypes = []
     for name, argtypes in _SIGNATURES.items():
         fn = getattr(lib, name, None)
         if fn is None:
@@ -100,3 +103,17 @@ def check_device() -> None:
     lib = load()
     if lib.pylon_check_device() != 0:
         raise KernelError(lib.pylon_last_error().decode(errors="replace"))
+
+
+_units: Optional[int] = None
+
+
+def compute_units() -> int:
+    """Compute units of the current device, asked of the runtime once."""
+    global _units
+    if _units is None:
+        units = load().pylon_compute_units()
+        if units <= 0:
+            raise KernelError("the number of compute units of the device is unknown (no GPU?)")
+        _units = units
+    return _units

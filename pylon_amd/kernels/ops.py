@@ -222,17 +222,17 @@ def decode_attention_ok(q: torch.Tensor, k_cache: torch.Tensor) -> bool:
             and n_heads % n_kv_heads == 0 and n_heads // n_kv_heads <= 16)
 
 
-def decode_splits(tokens: int, n_kv_heads: int, max_len: Optional[int]) -> int:
+def decode_splits(tokens: int, n_kv_heads: int, max_len: Optional[int], units: int = plan.UNITS) -> int:
     """Wavefronts (1, 2, 4 or 8) that share the keys of one (token, key/value head):
     ranges of about 64 keys (one batch of loads per wave) while the launch stays within a
     few thousand waves.  ``max_len`` is the most keys a workgroup gets (an upper bound
     under graph capture)."""
     waves = 8
-    if tokens * n_kv_heads > 256:
+    if tokens * n_kv_heads > units:
         # more workgroups than compute units: smaller ones run side by side (64 tokens of 140
         # keys: 13.8 us with four waves, 21.6 with eight; of 1,000 keys: 47 against 52)
         waves = 4
-    while waves > 1 and tokens * n_kv_heads * waves > 4096:
+    while waves > 1 and tokens * n_kv_heads * waves > 16 * units:
         waves //= 2
     if max_len is not None:
         while waves > 1 and (waves // 2) * 64 >= max_len:
@@ -248,19 +248,27 @@ def _like(q: torch.Tensor, out: Optional[torch.Tensor], name: str) -> torch.Tens
     return out
 
 
-def decode_cuts(tokens: int, n_kv_heads: int, max_len: Optional[int]) -> int:
+def decode_cuts(tokens: int, n_kv_heads: int, max_len: Optional[int], units: int = plan.UNITS) -> int:
     """Workgroups that share the keys of one (token, key/value head) before the waves of
     each share theirs: more than one when a few long requests would otherwise occupy a
-    fraction of the chip.  Measured on 256 compute units: about 256 workgroups in all, each
+    fraction of the chip.  Measured on 256 compute units: about one workgroup per unit, each
     with at least 1024 keys of ``max_len`` (which may be an upper bound well above the true
     lengths).  E.g. 8 tokens of 8192 keys: 53 us with 4 cuts, 102 us with one; more cuts
     than that lose again to the second kernel and its partial results."""
     cuts = 1
     if max_len is None:
         return cuts
-    while tokens * n_kv_heads * cuts * 2 <= 256 and max_len // (cuts * 2) >= 1024 and cuts < 64:
+    while tokens * n_kv_heads * cuts * 2 <= units and max_len // (cuts * 2) >= 1024 and cuts < 64:
         cuts *= 2
     return cuts
+
+
+def decode_launch(tokens: int, n_kv_heads: int, span: int) -> tuple:
+    """(cuts, splits) for decode attention of ``tokens`` single tokens that each see at most
+    ``span`` keys, on the current device."""
+    units = _lib.compute_units()
+    cuts = decode_cuts(tokens, n_kv_heads, span, units)
+    return cuts, decode_splits(tokens * cuts, n_kv_heads, -(-span // cuts), units)
 
 
 def _decode_scratch(tokens: int, n_heads: int, head_dim: int, n_cuts: int, device) -> Optional[torch.Tensor]:
@@ -537,7 +545,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.d
         if not x.is_cuda:
             raise KernelError("linear: operands must live on the GPU; there is no CPU path")
         if _streaming_ok(x, weight, STREAM_ROWS):
-            choice = plan.plan_projection(x.shape[0], *weight.shape)
+            choice = plan.plan_projection(x.shape[0], *weight.shape)  # no rule of it counts compute units
             if choice.kernel == "rows":
                 return gemm_rows(x, weight, out_dtype=out_dtype, col_tiles=choice.col_tiles, out=out)
             if choice.kernel == "skinny":
@@ -558,7 +566,7 @@ def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: tor
     result (:func:`plan.plan_residual`).  For more rows (prompt portions) it is the library's
     product rounded once to bfloat16."""
     if _streaming_ok(x, weight, STREAM_ROWS):
-        choice = plan.plan_residual(x.shape[0], *weight.shape)
+        choice = plan.plan_residual(x.shape[0], *weight.shape, units=_lib.compute_units())
         if choice.kernel == "rows":
             return gemm_rows(x, weight, out_dtype=torch.float32, parts=choice.parts, col_tiles=choice.col_tiles)
         if choice.kernel == "skinny":

@@ -18,7 +18,7 @@ from dataclasses import dataclass
 FEW_ROWS = 16      # one tile of rows of x
 STREAM_ROWS = 64   # most rows of x a weight-streaming kernel takes
 TALL = 32768       # a matrix of at least this many rows (a vocabulary head) is "tall"
-UNITS = 256        # compute units
+UNITS = 256        # compute units of an MI355X; callers on a device pass its own count
 
 
 @dataclass(frozen=True)
@@ -38,26 +38,26 @@ def aliased_rows(k: int) -> bool:
     return k % 4096 == 0
 
 
-def rows_split(n: int, k: int, rows: int = STREAM_ROWS) -> tuple:
+def rows_split(n: int, k: int, rows: int = STREAM_ROWS, units: int = UNITS) -> tuple:
     """(parts, col_tiles) of the rows kernel for a product into the residual stream.
     Workgroups of 128 columns for deep matrices (beyond 16 rows, where the rows of x weigh
     more, from a depth of 8192) and for wide ones, else of 64; K cut into the largest power of
-    two of parts (at most 16, of at least 256 elements each) that keeps the workgroups at 256
-    or fewer, one per compute unit: more of them only re-read the rows of x."""
+    two of parts (at most 16, of at least 256 elements each) that keeps the workgroups at one
+    per compute unit or fewer: more of them only re-read the rows of x."""
     col_tiles = 2 if (k >= 8192 and rows > FEW_ROWS) or k >= 16384 or n > 4096 else 1
     groups = -(-n // (64 * col_tiles))
     parts = 1
-    while parts < 16 and 2 * parts * groups <= UNITS and k // (2 * parts) >= 256:
+    while parts < 16 and 2 * parts * groups <= units and k // (2 * parts) >= 256:
         parts *= 2
     return parts, col_tiles
 
 
-def skinny_parts(n: int, k: int) -> int:
+def skinny_parts(n: int, k: int, units: int = UNITS) -> int:
     """Ranges the skinny kernel cuts K into so that a matrix of few rows still fills the chip
     (at most 4: with 8 a whole decode step measured 7 % slower)."""
     tiles = (n + 15) // 16
     parts = 1
-    while tiles * parts < 512 and parts < 4 and k // (parts * 2) >= 512:
+    while tiles * parts < 2 * units and parts < 4 and k // (parts * 2) >= 512:
         parts *= 2
     return parts
 
@@ -71,17 +71,17 @@ def deep_or_narrow(n: int, k: int) -> bool:
     return k >= 2 * n or n <= 4096
 
 
-def plan_residual(rows: int, n: int, k: int) -> Product:
+def plan_residual(rows: int, n: int, k: int, units: int = UNITS) -> Product:
     """A product about to be added to the float32 residual stream (out and down projections),
     ``rows`` <= 64: float32 sums, never rounded, from whichever kernel.  Up to 16 rows the rows
     kernel also beats the skinny one (2560x4096 at 8 rows: 6.2 against 8.3 us, 2560x9728 11.5
     against 13.8, 5120x8192 20 against 23, 5120x25600 52 against 65)."""
     few = rows <= FEW_ROWS
     if deep_or_narrow(n, k) or (few and n <= 8192):
-        parts, col_tiles = rows_split(n, k, rows)
+        parts, col_tiles = rows_split(n, k, rows, units)
         return Product("rows", parts, col_tiles)
     if few:
-        return Product("skinny", skinny_parts(n, k))
+        return Product("skinny", skinny_parts(n, k, units))
     return Product("library")
 
 

@@ -58,8 +58,7 @@ class Attention(Part):
                 qkv, cache.k, tokens=tokens, n_heads=spec.n_heads, head_dim=spec.head_dim,
                 rot_dim=rotary[1] if rotary else 0):
             # one launch norms and rotates q and k, stores k and v, and attends
-            cuts = ops.decode_cuts(tokens, spec.n_kv_heads, self._span(ctx))
-            splits = ops.decode_splits(tokens * cuts, spec.n_kv_heads, -(-self._span(ctx) // cuts))
+            cuts, splits = ops.decode_launch(tokens, spec.n_kv_heads, self._span(ctx))
             context = ops.attention_decode_fused(
                 qkv, cache.k, cache.v, cache.block_table, None, ctx.positions,
                 n_heads=spec.n_heads, q_weight=self.params.get("q_norm"), k_weight=self.params.get("k_norm"),
@@ -79,8 +78,7 @@ class Attention(Part):
             positions=ctx.positions, slot_map=cache.slot_map, store_kv=stores,
         )
         if ctx.decode_only and ops.decode_attention_ok(q, cache.k):
-            cuts = ops.decode_cuts(tokens, spec.n_kv_heads, self._span(ctx))
-            splits = ops.decode_splits(tokens * cuts, spec.n_kv_heads, -(-self._span(ctx) // cuts))
+            cuts, splits = ops.decode_launch(tokens, spec.n_kv_heads, self._span(ctx))
             # in a decode-only step token t is row t
             context = ops.attention_decode(
                 q, cache.k, cache.v, cache.block_table, None, ctx.positions,
@@ -99,8 +97,7 @@ class Attention(Part):
                 span = int(ctx.starts[:singles].max()) + 1
                 if spec.window is not None:
                     span = min(span, spec.window)
-                cuts = ops.decode_cuts(singles, spec.n_kv_heads, span)
-                splits = ops.decode_splits(singles * cuts, spec.n_kv_heads, -(-span // cuts))
+                cuts, splits = ops.decode_launch(singles, spec.n_kv_heads, span)
                 ops.attention_decode(
                     q[:singles], cache.k, cache.v, cache.block_table, None, ctx.positions[:singles],
                     page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits,

@@ -1,0 +1,158 @@
+"""Every matrix product a step of the published Qwen3 dense sizes runs, at its real size,
+through the dispatchers the parts call (``ops.linear``, ``ops.linear_for_residual``,
+``ops.linear_glu``), against a float64 product: which kernel the plan picks for the case,
+how that kernel is laid over the chip, and the numbers.
+
+The vocabulary head is /root/reference/src/pylon/model/model.py:140-144, q/k/v and the out
+projection /root/reference/src/pylon/model/layers.py:126,138, gate/up and down :26-27.
+
+Kernel instance reached per case (``gemm_rows_kernel<MT, CT, GLU, WAVES, TO>`` with MT =
+ceil(rows / 16); "spread": the waves of a workgroup take column groups one per compute unit
+apart; ``groups x parts`` workgroups):
+
+=========  =====================  ======================================  ===================
+product    1, 8, 16 rows          17, 48, 64 rows                         65, 130 rows
+=========  =====================  ======================================  ===================
+4b qkv     rows CT1 2 waves,      library, bfloat16                       library, bfloat16
+           256x1 spread
+4b out     rows CT1 4w 40x4       rows CT1 4w 40x4                        library, bfloat16
+4b gate/up rows GLU 4w 256x1      rows GLU 4w 256x1 spread                library + silu_gate
+           spread
+4b down    rows CT1 4w 40x4       rows CT2 4w 20x8                        library, bfloat16
+4b head    rows CT2 4w 1187x1     rows CT2 4w 1187x1                      library, float32
+8b qkv     rows CT1 2w 256x1      library                                 library
+           spread
+8b out     rows CT1 4w 64x4       rows CT1 4w 64x4                        library
+8b gate/up skinny GLU             rows GLU 4w 256x1 spread                library + silu_gate
+8b down    rows CT1 4w 64x4       rows CT2 4w 32x8                        library
+8b head    skinny                 rows CT2 4w 1187x1                      library, float32
+32b qkv    rows CT1 4w 256x1      library                                 library
+           spread
+32b out    rows CT2 4w 40x4       library, float32                        library
+32b g/u    rows GLU 4w 400x1      library float32 + silu_gate             library + silu_gate
+32b down   rows CT2 4w 40x4       rows CT2 4w 40x4                        library
+32b head   rows CT2 4w 1187x1     rows CT2 4w 1187x1                      library, float32
+=========  =====================  ======================================  ===================
+"""
+import ctypes
+import zlib
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+VOCAB = 151936
+# (hidden, q width, key/value width, feed-forward width)
+SIZES = {"4b": (2560, 4096, 1024, 9728), "8b": (4096, 4096, 1024, 12288), "32b": (5120, 8192, 1024, 25600)}
+ROWS = (1, 8, 16, 17, 48, 64, 65, 130)
+
+# (kernel, parts, col_tiles, (waves, groups, spread)) for few (<= 16) and many (17..64) rows
+R = "rows"
+EXPECT = {
+    ("4b", "qkv"): ((R, 1, 1, (2, 256, 1)), ("library",)),
+    ("4b", "out"): ((R, 4, 1, (4, 40, 0)), (R, 4, 1, (4, 40, 0))),
+    ("4b", "gate_up"): ((R, 1, 2, (4, 256, 1)), (R, 1, 2, (4, 256, 1))),
+    ("4b", "down"): ((R, 4, 1, (4, 40, 0)), (R, 8, 2, (4, 20, 0))),
+    ("4b", "head"): ((R, 1, 2, (4, 1187, 0)), (R, 1, 2, (4, 1187, 0))),
+    ("8b", "qkv"): ((R, 1, 1, (2, 256, 1)), ("library",)),
+    ("8b", "out"): ((R, 4, 1, (4, 64, 0)), (R, 4, 1, (4, 64, 0))),
+    ("8b", "gate_up"): (("skinny",), (R, 1, 2, (4, 256, 1))),
+    ("8b", "down"): ((R, 4, 1, (4, 64, 0)), (R, 8, 2, (4, 32, 0))),
+    ("8b", "head"): (("skinny",), (R, 1, 2, (4, 1187, 0))),
+    ("32b", "qkv"): ((R, 1, 1, (4, 256, 1)), ("library",)),
+    ("32b", "out"): ((R, 4, 2, (4, 40, 0)), ("library",)),
+    ("32b", "gate_up"): ((R, 1, 2, (4, 400, 0)), ("library",)),
+    ("32b", "down"): ((R, 4, 2, (4, 40, 0)), (R, 4, 2, (4, 40, 0))),
+    ("32b", "head"): ((R, 1, 2, (4, 1187, 0)), (R, 1, 2, (4, 1187, 0))),
+}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from pylon_amd.kernels import check_device, ops as _ops
+
+    check_device()
+    return _ops
+
+
+def shape_of(model: str, product: str):
+    hidden, q, kv, inter = SIZES[model]
+    return {"qkv": (q + 2 * kv, hidden), "out": (hidden, q), "gate_up": (2 * inter, hidden),
+            "down": (hidden, inter), "head": (VOCAB, hidden)}[product]
+
+
+def launch_shape(n, ldw, parts, col_tiles, glu):
+    from pylon_amd.kernels import library
+
+    out = (ctypes.c_int * 3)()
+    assert library.load().pylon_gemm_rows_shape(n, ldw, parts, col_tiles, glu, 0, 0, out) == 0
+    return tuple(out)
+
+
+def chosen(model, product, rows, units):
+    """What the plan picks for this case, in the form of EXPECT's entries."""
+    from pylon_amd.kernels import plan
+
+    n, k = shape_of(model, product)
+    if product in ("out", "down"):
+        c = plan.plan_residual(rows, n, k, units=units)
+    elif product == "gate_up":
+        c = plan.plan_gated(rows, n // 2, k, k)
+    else:
+        c = plan.plan_projection(rows, n, k)
+    if c.kernel != "rows":
+        return (c.kernel,)
+    glu = product == "gate_up"
+    return (c.kernel, c.parts, c.col_tiles, launch_shape(n // 2 if glu else n, k, c.parts, c.col_tiles, int(glu)))
+
+
+@pytest.mark.parametrize("product", ["qkv", "out", "gate_up", "down", "head"])
+@pytest.mark.parametrize("model", list(SIZES))
+def test_a_product_at_its_real_size(ops, model, product):
+    from pylon_amd.kernels import library
+
+    n, k = shape_of(model, product)
+    gen = torch.Generator(device=DEV).manual_seed(zlib.crc32(f"{model}/{product}".encode()))
+    w = (torch.randn((n, k), generator=gen, device=DEV) * 0.02).to(torch.bfloat16)
+    x = torch.randn((max(ROWS), k), generator=gen, device=DEV).to(torch.bfloat16)
+    want = torch.mm(x.double(), w.double().t())
+    if product == "gate_up":
+        g, u = want[:, : n // 2], want[:, n // 2:]
+        want = g / (1 + torch.exp(-g)) * u
+    want = want.cpu().numpy()
+    del gen
+    few, many = EXPECT[(model, product)]
+    units = library.compute_units()
+    assert units == 256  # the expectations above are those of an MI355X
+    for rows in ROWS:
+        if rows <= 64:
+            assert chosen(model, product, rows, units) == (few if rows <= 16 else many), (model, product, rows)
+        xr = x[:rows].contiguous()
+        if product in ("out", "down"):
+            got = ops.linear_for_residual(xr, w, out_dtype=torch.bfloat16)
+            if rows <= 64:  # float32 sums, never rounded: whole, or K cut into parts
+                assert got.dtype == torch.float32
+                got = got.sum(0, dtype=torch.float64) if got.dim() == 3 else got
+            else:
+                assert got.dtype == torch.bfloat16
+        elif product == "gate_up":
+            got = ops.linear_glu(xr, w, out_dtype=torch.bfloat16)
+            assert got.dtype == torch.bfloat16
+        elif product == "head":
+            got = ops.linear(xr, w, out_dtype=torch.float32)  # logits: float32 at every row count
+            assert got.dtype == torch.float32
+        else:
+            got = ops.linear(xr, w, out_dtype=torch.bfloat16)
+        ref = want[:rows]
+        assert got.shape == ref.shape, (model, product, rows, tuple(got.shape))
+        scale = np.abs(ref).max()
+        # float32 sums: a few ulps of accumulated rounding; bfloat16: one rounding of the result
+        # (2^-9), and a second one where the library rounds gate and up before the activation
+        bound = 2e-6 if got.dtype != torch.bfloat16 else (1.2e-2 if product == "gate_up" and rows > 64 else 6e-3)
+        error = np.abs(got.double().cpu().numpy() - ref).max()
+        assert error <= bound * scale, (model, product, rows, error / scale)

@@ -55,34 +55,12 @@ def folders(tmp_path_factory):
 
 def run_steps(folder, dtype, steps, *, page_size=64, max_tokens=None, vocab):
     """Drive Runner.step with the trace, the way the replay program does."""
-    from pylon_amd.engine import Runner, StepEntry
+    from pylon_amd.engine import Runner
 
     max_tokens = max_tokens or traces.peak_tokens(steps, page_size)
     runner = Runner.from_folder(folder, dtype=dtype, page_size=page_size,
                                 num_pages=-(-max_tokens // page_size), max_requests=8)
-    live, outputs = {}, {}
-    reused = set()
-    handed = set()
-    for step in steps:
-        entries = []
-        for e in step["entries"]:
-            if e["id"] not in live:
-                live[e["id"]] = runner.open(e["id"])
-            entries.append(StepEntry(live[e["id"]], e["tokens"], e["want"]))
-        logits = runner.step(entries)
-        for e in step["entries"]:
-            for page in live[e["id"]].pages[0]:
-                if (e["id"], page) not in handed:
-                    if any(p == page for _, p in handed):
-                        reused.add(page)
-                    handed.add((e["id"], page))
-        if logits is not None:
-            outputs[step["step"]] = logits.cpu().numpy()
-        for rid in step["end"]:
-            runner.close(live.pop(rid))
-        runner.manager.check()
-    assert not runner.manager.live_sequences()
-    return traces.collect(steps, outputs, vocab), reused
+    return traces.replay(runner, steps, vocab)
 
 
 def check(got, want, dtype, what):
@@ -182,7 +160,8 @@ def test_a_refused_step_leaves_the_cache_as_it_was(folders):
         runner.step([StepEntry(b, [1] * 129, [])])
     rest = runner.step([StepEntry(a, toks[40:], list(range(len(toks) - 40)))]).cpu().numpy()
     got = np.concatenate([first, rest])
-    assert np.abs(got - want["r3"]).max() <= BOUND["float32"] * np.abs(want["r3"]).max()
+    ok, row, frac = rows_within(got, want["r3"], BOUND["float32"])
+    assert ok, f"position {row} is off by {frac:.3e} of its largest logit"
     runner.manager.check()
 
 
@@ -223,5 +202,5 @@ def test_replay_program_as_a_user_runs_it(folders, tmp_path, dtype):
         if skipped == len(ref):
             assert rid not in got  # all of it ran in the step that asked for nothing
             continue
-        scale = np.abs(ref).max()
-        assert np.abs(got[rid] - ref[skipped:]).max() <= BOUND[dtype] * scale, rid
+        ok, row, frac = rows_within(got[rid], ref[skipped:], BOUND[dtype])
+        assert ok, f"{rid}: position {skipped + row} is off by {frac:.3e} of its largest logit"

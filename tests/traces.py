@@ -111,3 +111,33 @@ def collect(steps: List[dict], outputs: Dict[int, "object"], vocab: int):
             seen[e["id"]] = start + len(e["tokens"])
         assert out is None or cursor == out.shape[0]
     return {rid: np.stack([r[i] for i in sorted(r)]) for rid, r in rows.items()}
+
+
+def replay(runner, steps: List[dict], vocab: int, idle: int = 0):
+    """Drive ``runner.step`` with the trace, the way the replay program does.  Returns
+    ({request: logits by position}, the pages that more than one request held in turn).
+    ``idle``: requests the caller keeps open beside the trace's."""
+    from pylon_amd.engine import StepEntry
+
+    live, outputs = {}, {}
+    reused, handed = set(), set()
+    for step in steps:
+        entries = []
+        for e in step["entries"]:
+            if e["id"] not in live:
+                live[e["id"]] = runner.open(e["id"])
+            entries.append(StepEntry(live[e["id"]], e["tokens"], e["want"]))
+        logits = runner.step(entries)
+        for e in step["entries"]:
+            for page in live[e["id"]].pages[0]:
+                if (e["id"], page) not in handed:
+                    if any(p == page for _, p in handed):
+                        reused.add(page)
+                    handed.add((e["id"], page))
+        if logits is not None:
+            outputs[step["step"]] = logits.cpu().numpy()
+        for rid in step["end"]:
+            runner.close(live.pop(rid))
+        runner.manager.check()
+    assert len(runner.manager.live_sequences()) == idle
+    return collect(steps, outputs, vocab), reused
