@@ -4,16 +4,23 @@ and uniform-random token ids, on one MI355X.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
                     [--shape 4b|8b|32b] [--prompt-len N]
 
-A "step" is one decode step: one token for each of ``batch`` running requests through
-the step function, then greedy sampling on the device and the copy of the chosen ids to
-the host.  As in the engine's ticks, a step is queued before the host has read the ids of
-the step before it (they are fed back on the device), and every step's ids are read.  ``value`` is decoded tokens per second at the default batch of 8.  The same
-line carries the prefill of 2,048 tokens, the decode step's share of the HBM roofline,
-decode rates at batch 1 and 64, and two rates through the scheduler (queueing, admission and
-the prompts' prefill included): ``points.engine_b8`` with the same 128-token prompts and 512
-new tokens, ``points.engine_prefill_heavy_b8`` with 2,048-token prompts and 32 new tokens.
-``--shape`` and ``--prompt-len`` measure the same at the Qwen3-8B and 32B layer sizes and
-at longer contexts; the default run is the 4B shape with 128-token prompts.
+Everything goes the product's own way.  Start-up is ``Runner.from_random``: the fit check,
+the measured activation headroom, the page pool sized from the card's memory and the decode
+graphs captured before serving, as ``main.py generate --random`` does it.  Requests go through
+``Engine``: queue, admission, prompts cut into portions of at most 2,048 tokens, ticks.
+
+A "step" is one tick of the engine once all ``batch`` requests decode: one token for each of
+them through the step function (replayed from a HIP graph), greedy sampling on the device, and
+the read of the chosen ids by the host; as in serving, a tick queues its step before it reads
+the ids of the step before (they are fed back on the device).  ``value`` is decoded tokens per
+second at the default batch of 8.  The same line carries the prefill of 2,048 tokens (one
+request from its arrival to its first token), the decode step's share of the HBM roofline, and
+under ``points`` decode rates at batch 1 and 64, at contexts of 4,096 and 8,000 tokens, a prompt
+of 8,191 tokens in four portions, a step of 64 decoded tokens beside a 2,048-token portion, and
+two rates over whole requests (queueing, admission and prefill included): ``engine_b8`` with the
+same 128-token prompts and 512 new tokens, ``engine_prefill_heavy_b8`` with 2,048-token prompts
+and 32 new tokens.  ``--shape`` and ``--prompt-len`` measure the same at the Qwen3-8B and 32B
+layer sizes and at longer contexts.
 """
 from __future__ import annotations
 
@@ -52,6 +59,7 @@ PAGE_SIZE = 256
 PROMPT_LEN = 128
 NEW_TOKENS = 512
 PREFILL_TOKENS = 2048
+MOST_NEW_TOKENS = 2048  # what a request may ask for (Sampling's range, the reference's)
 # The reference's own published figure for this workload (128-token prompts, 512 new tokens,
 # 8 requests at a time, Qwen3-4B): 199.8 output tokens/s, through its server on one NVIDIA L4
 # (/root/reference/README.md:73).  Other hardware: the ratio says how far apart the two
@@ -65,23 +73,11 @@ def config_json(shape: dict, layers: int) -> dict:
     return cfg
 
 
-def build_runner(shape: dict, layers: int, dtype: str, max_requests: int, num_pages: int, graphs: bool):
-    import torch
+def serving_config(dtype: str, max_batch: int, graphs: bool, **more):
+    from pylon_amd.config import PylonConfig
 
-    from pylon_amd.config import resolve
-    from pylon_amd.engine import Model, Runner, resolve_dtype
-    from pylon_amd.weights import fill_random_model
-
-    raw = config_json(shape, layers)
-    arch = resolve(raw)
-    cfg = arch.parse_config(raw)
-    model = Model(arch.model_spec(cfg), dtype=resolve_dtype(dtype), device="cuda:0")
-    fill_random_model(model, arch, cfg, seed=0, std=0.02)  # the random-weights mode, on the device
-    runner = Runner(model, page_size=PAGE_SIZE, num_pages=num_pages, max_requests=max_requests)
-    if graphs:
-        runner.enable_graphs(max_requests, max_tokens_per_request=shape["max_position_embeddings"])
-    torch.cuda.synchronize()
-    return runner, cfg
+    return PylonConfig(dtype=dtype, max_batch_size=max_batch, max_queue_size=max(max_batch, 1), page_size=PAGE_SIZE,
+                       prefill_chunk_size=PREFILL_TOKENS, cuda_graphs=graphs, **more)
 
 
 def weight_bytes(runner) -> int:
@@ -103,155 +99,156 @@ def linear_flops_per_token(cfg) -> float:
     return 2.0 * cfg.num_hidden_layers * per_layer
 
 
-def feed_prompts(runner, sampler, seqs, prompts) -> None:
-    """The prompts through the step function in steps of at most PREFILL_TOKENS tokens, cut by
-    the scheduler's own rule (:func:`pylon_amd.engine.scheduler.cut_prompts`: short prompts
-    side by side, a long one in portions); the first new token of each request is chosen on
-    the device."""
-    from pylon_amd.engine import StepEntry
-    from pylon_amd.engine.scheduler import PromptWork, cut_prompts
+def attention_flops(cfg, new_tokens: int, cached: int = 0) -> float:
+    """Score and value products of ``new_tokens`` tokens that follow ``cached`` ones (causal)."""
+    pairs = new_tokens * cached + new_tokens * (new_tokens + 1) / 2
+    return 4.0 * cfg.num_hidden_layers * cfg.num_attention_heads * cfg.head_dim * pairs
+
+
+class Serving:
+    """``batch`` requests of ``prompt_len`` random ids each, brought through the engine to the
+    point where every one of them decodes; then ticks can be timed."""
+
+    def __init__(self, runner, cfg, args, batch: int, prompt_len: int, ticks: int, seed: int, room: int = 0):
+        import numpy as np
+
+        from pylon_amd.engine.engine import Engine
+        from pylon_amd.sampling import Sampling
+
+        self.runner, self.cfg, self.batch = runner, cfg, batch
+        self.rng = np.random.default_rng(seed)
+        config = serving_config(args.dtype, batch + room, runner.graphs is not None)
+        self.engine = Engine(config, runner=runner)
+        # the prompts' portions take ticks in which the first requests already decode
+        prefill_ticks = -(-batch * prompt_len // PREFILL_TOKENS) + 2
+        limit = runner.model.spec.max_positions - prompt_len
+        self.new_tokens = min(MOST_NEW_TOKENS, limit, ticks + prefill_ticks + 8)
+        self.ticks = self.new_tokens - prefill_ticks - 8
+        if self.ticks < 1:
+            raise SystemExit(f"bench.py: {prompt_len}-token prompts leave no room for decode steps")
+        sampling = Sampling(max_new_tokens=self.new_tokens, temperature=0.0)
+        self.futures = [self.engine.enqueue(self.rng.integers(0, cfg.vocab_size, prompt_len).tolist(), None, sampling)
+                        for _ in range(batch)]
+        while True:
+            self.engine.tick()
+            decoding, portions = self.engine.last_step
+            if len(decoding) == batch and not portions:
+                break
+
+    def timed_ticks(self, count: int, warmup: int):
+        """(seconds, mean cached tokens read per step over all rows) of ``count`` ticks."""
+        import torch
+
+        if warmup + count > self.ticks:
+            raise SystemExit(f"bench.py: {warmup} + {count} steps do not fit the requests' {self.ticks} decode ticks")
+        for _ in range(warmup):
+            self.engine.tick()
+        self.ticks -= warmup + count
+        seqs = self.runner.manager.live_sequences()
+        torch.cuda.synchronize()
+        context = 0
+        started = time.perf_counter()
+        for _ in range(count):
+            context += sum(s.length + 1 for s in seqs)
+            self.engine.tick()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        decoding, portions = self.engine.last_step
+        assert len(decoding) == self.batch and not portions and self.engine.steps_run >= count
+        return elapsed, context / count
+
+    def mixed_tick_ms(self, repeats: int) -> float:
+        """Milliseconds of device time of a step that carries every decoding request's token
+        beside a PREFILL_TOKENS portion of a new prompt (median): events around the tick that
+        queues it.  The engine must have been made with ``room=1``."""
+        import torch
+
+        from pylon_amd.sampling import Sampling
+
+        times = []
+        for _ in range(repeats + 1):
+            prompt = self.rng.integers(0, self.cfg.vocab_size, PREFILL_TOKENS).tolist()
+            future = self.engine.enqueue(prompt, None, Sampling(max_new_tokens=1, temperature=0.0))
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            self.engine.tick()
+            end.record()
+            decoding, portions = self.engine.last_step
+            assert len(decoding) == self.batch and [count for _, count in portions] == [PREFILL_TOKENS]
+            while not future.done():
+                self.engine.tick()
+            self.ticks -= 3
+            end.synchronize()
+            times.append(start.elapsed_time(end))
+        times = sorted(times[1:])
+        return times[len(times) // 2]
+
+    def finish(self) -> None:
+        self.engine.run_until_idle()
+        results = [f.result(timeout=0) for f in self.futures]
+        assert all(len(r.output_ids) == self.new_tokens for r in results)
+        self.engine.close()
+
+
+def decode_point(runner, cfg, args, batch: int, prompt_len: int, steps: int, seed: int, mixed: bool = False) -> dict:
+    """Tokens per second and roofline share of decode steps of ``batch`` requests at this context."""
+    serving = Serving(runner, cfg, args, batch, prompt_len, steps + args.warmup + (24 if mixed else 0), seed,
+                      room=1 if mixed else 0)
+    elapsed, context = serving.timed_ticks(steps, args.warmup)
+    out = {"tokens_per_s": batch * steps / elapsed, "ms": 1e3 * elapsed / steps,
+           "bytes": weight_bytes(runner) + context * runner.manager.bytes_per_token, "context": context / batch}
+    out["frac"] = out["bytes"] / (elapsed / steps) / HBM_BYTES_PER_S
+    if mixed:
+        out["mixed_ms"] = serving.mixed_tick_ms(repeats=5)
+    serving.finish()
+    return out
+
+
+def prefill_run(runner, cfg, args, tokens: int, repeats: int, seed: int) -> float:
+    """Seconds from a request's arrival to its first token, for one prompt of ``tokens`` random
+    ids and nothing else running (portions of at most PREFILL_TOKENS); the median."""
+    import numpy as np
+    import torch
+
+    from pylon_amd.engine.engine import Engine
     from pylon_amd.sampling import Sampling
 
-    fed = [0] * len(seqs)
-    while True:
-        work = [PromptWork(i, len(prompts[i]) - fed[i], 0.0) for i in range(len(seqs)) if fed[i] < len(prompts[i])]
-        portions = cut_prompts(work, PREFILL_TOKENS, 0.0)
-        if not portions:
-            return
-        entries = []
-        for i, take in portions:
-            last = fed[i] + take == len(prompts[i])
-            entries.append(StepEntry(seqs[i], prompts[i][fed[i]: fed[i] + take], [take - 1] if last else []))
-            fed[i] += take
-        out = runner.step(entries)
-        wanted = sum(len(e.want) for e in entries)
-        if wanted:
-            greedy = [(Sampling(temperature=0.0), 0)] * wanted
-            sampler.launch(out, greedy, chosen=runner.chosen, place=runner.logit_slots).result()
-
-
-def decode_run(runner, cfg, batch: int, steps: int, warmup: int, seed: int, prompt_len: int = PROMPT_LEN):
-    """Prefill ``batch`` prompts of ``prompt_len`` random ids, then time ``steps`` decode steps."""
-    import numpy as np
-    import torch
-
-    from pylon_amd.engine import PENDING, StepEntry
-    from pylon_amd.sampling import Sampler, Sampling
-
-    sampler = Sampler(runner.model.device)
-    greedy = [(Sampling(temperature=0.0), 0)] * batch
     rng = np.random.default_rng(seed)
-    seqs = [runner.open(f"b{batch}-{i}") for i in range(batch)]
-    prompts = [rng.integers(0, cfg.vocab_size, prompt_len).tolist() for _ in range(batch)]
-    feed_prompts(runner, sampler, seqs, prompts)
-
-    entries = [StepEntry(seqs[i], [PENDING], [0]) for i in range(batch)]
-    produced = []
-
-    def one_step(before):
-        out = runner.step(entries)
-        draw = sampler.launch(out, greedy, chosen=runner.chosen, place=runner.logit_slots)
-        if before is not None:
-            produced.append(before.result())
-        return draw
-
-    draw = None
-    for _ in range(warmup):
-        draw = one_step(draw)
-    torch.cuda.synchronize()
-    context_sum = 0
-    started = time.perf_counter()
-    for _ in range(steps):
-        context_sum += sum(s.length + 1 for s in seqs)
-        draw = one_step(draw)
-    produced.append(draw.result())
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - started
-    assert len(produced) == warmup + steps and all(len(p) == batch for p in produced)
-    for s in seqs:
-        runner.close(s)
-    return elapsed, context_sum / steps  # seconds, mean cached tokens read per step (all rows)
-
-
-def prefill_run(runner, cfg, repeats: int, seed: int):
-    """One prompt of PREFILL_TOKENS random ids in one step; the median of ``repeats`` runs."""
-    import numpy as np
-    import torch
-
-    from pylon_amd.engine import StepEntry
-
-    rng = np.random.default_rng(seed)
+    engine = Engine(serving_config(args.dtype, 1, runner.graphs is not None), runner=runner)
     times = []
-    for r in range(repeats + 1):
-        seq = runner.open(f"prefill-{r}")
-        prompt = rng.integers(0, cfg.vocab_size, PREFILL_TOKENS).tolist()
+    for _ in range(repeats + 1):
+        prompt = rng.integers(0, cfg.vocab_size, tokens).tolist()
         torch.cuda.synchronize()
         started = time.perf_counter()
-        out = runner.step([StepEntry(seq, prompt, [PREFILL_TOKENS - 1])])
-        out.cpu()
+        result, = engine.generate([prompt], Sampling(max_new_tokens=1, temperature=0.0))
         times.append(time.perf_counter() - started)
-        runner.close(seq)
+        assert len(result.output_ids) == 1
+    engine.close()
     times = sorted(times[1:])  # the first run warms the library's kernels up
     return times[len(times) // 2]
 
 
-def mixed_run(runner, cfg, batch: int, prompt_len: int, repeats: int, seed: int) -> float:
-    """Seconds of one mixed step: one token for each of ``batch`` requests that hold
-    ``prompt_len`` tokens, beside a PREFILL_TOKENS portion of a new prompt, with greedy
-    sampling of the batch + 1 wanted rows on the device; the median."""
+def engine_run(runner, cfg, args, batch: int, seed: int, prompt_len: int = PROMPT_LEN, new_tokens: int = NEW_TOKENS):
+    """Whole requests: ``batch`` requests of ``prompt_len`` random ids and ``new_tokens`` greedy
+    tokens each, queued at once; generated tokens per second from the first request's arrival
+    to the last one's end (admission, the prompts' prefill, ticks, sampling and the host's
+    reading of every token included), and the median time from a request's arrival to its
+    first token in milliseconds."""
     import numpy as np
     import torch
 
-    from pylon_amd.engine import StepEntry
-    from pylon_amd.sampling import Sampler, Sampling
-
-    rng = np.random.default_rng(seed)
-    sampler = Sampler(runner.model.device)
-    greedy = [(Sampling(temperature=0.0), 0)] * (batch + 1)
-    seqs = [runner.open(f"m{batch}-{i}") for i in range(batch)]
-    feed_prompts(runner, sampler, seqs, [rng.integers(0, cfg.vocab_size, prompt_len).tolist() for _ in seqs])
-    times = []
-    for r in range(repeats + 1):
-        fresh = runner.open(f"mixed-prompt-{r}")
-        entries = [StepEntry(s, [int(rng.integers(0, cfg.vocab_size))], [0]) for s in seqs]
-        entries.append(StepEntry(fresh, rng.integers(0, cfg.vocab_size, PREFILL_TOKENS).tolist(), [PREFILL_TOKENS - 1]))
-        torch.cuda.synchronize()
-        started = time.perf_counter()
-        out = runner.step(entries)
-        sampler.launch(out, greedy, chosen=runner.chosen, place=runner.logit_slots).result()
-        times.append(time.perf_counter() - started)
-        runner.close(fresh)
-    for s in seqs:
-        runner.close(s)
-    times = sorted(times[1:])
-    return times[len(times) // 2]
-
-
-def engine_run(runner, cfg, batch: int, seed: int, prompt_len: int = PROMPT_LEN, new_tokens: int = NEW_TOKENS):
-    """The same work through the scheduler: ``batch`` requests of ``prompt_len`` random ids and
-    ``new_tokens`` greedy tokens each, queued at once; generated tokens per second from the
-    first request's arrival to the last one's end (admission, the prompts' prefill, ticks,
-    sampling and the host's reading of every token included), and the median time from a
-    request's arrival to its first token in milliseconds."""
-    import numpy as np
-    import torch
-
-    from pylon_amd.config import PylonConfig
     from pylon_amd.engine.engine import Engine
     from pylon_amd.sampling import Sampling
 
     rng = np.random.default_rng(seed)
     prompts = [rng.integers(0, cfg.vocab_size, prompt_len).tolist() for _ in range(batch)]
-    engine = Engine(PylonConfig(max_batch_size=batch, max_queue_size=batch, page_size=PAGE_SIZE), runner=runner)
+    engine = Engine(serving_config(args.dtype, batch, runner.graphs is not None), runner=runner)
     sampling = Sampling(max_new_tokens=new_tokens, temperature=0.0)
-    if runner.graphs is not None:  # as a server does at start-up
-        longest = prompt_len + new_tokens
-        runner.capture_graphs(range(1, batch + 1),
-                              bounds=[b for b in runner.graphs.bounds() if b < 2 * longest])
     torch.cuda.synchronize()
     started = time.perf_counter()
     results = engine.generate(prompts, sampling)
     elapsed = time.perf_counter() - started
+    engine.close()
     assert all(len(r.output_ids) == new_tokens for r in results)
     first = sorted(r.first_token_seconds for r in results)
     return batch * new_tokens / elapsed, 1e3 * first[len(first) // 2]
@@ -298,7 +295,7 @@ def main() -> int:
     parser.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens cached before decoding starts")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
-    parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    parser.add_argument("--no-points", action="store_true", help="skip the other batch sizes and contexts")
     parser.add_argument("--no-prefill", action="store_true")
     parser.add_argument("--no-peaks", action="store_true", help="skip the probes of this device's own peaks")
     parser.add_argument("--mixed", action="store_true",
@@ -314,35 +311,34 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: A GPU is required.", file=sys.stderr)
         return 1
+    from pylon_amd.engine import Runner
 
     shape = SHAPES[args.shape]
     layers = args.layers or shape["num_hidden_layers"]
     context_length = shape["max_position_embeddings"]
     prompt_len = args.prompt_len
-    steps = min(args.steps, context_length - prompt_len - args.warmup)
-    max_batch = args.batch if args.no_points else max(64, args.batch)
-    # The pool holds a whole context for every request where that stays under a third of the
-    # card's memory, else what the longest run here needs.
-    element = 2 if args.dtype == "bfloat16" else 4
-    page_bytes = 2 * layers * PAGE_SIZE * shape["num_key_value_heads"] * shape["head_dim"] * element
-    pages_per_request = context_length // PAGE_SIZE
-    if max_batch * pages_per_request * page_bytes > 100e9:
-        longest = max(prompt_len + steps + args.warmup + 1, PREFILL_TOKENS)
-        pages_per_request = -(-longest // PAGE_SIZE) + 1
-    runner, cfg = build_runner(shape, layers, args.dtype, max_requests=max_batch + 1,
-                               num_pages=(max_batch + 1) * pages_per_request, graphs=not args.no_graphs)
+    max_batch = args.batch + 1 if args.no_points else max(64, args.batch) + 1
+    # The product's start-up: weights drawn in place, the pool sized from the card's memory
+    # under the serving options (at most max_batch requests of the longest length), graphs.
+    raw = config_json(shape, layers)
+    runner = Runner.from_random(raw, 0, serving_config(args.dtype, max_batch, not args.no_graphs), std=0.02)
+    cfg = runner.config
     dtype_key = "bf16" if args.dtype == "bfloat16" else "fp32"
     if args.prefill_only:
-        seconds = prefill_run(runner, cfg, repeats=5, seed=2)
+        seconds = prefill_run(runner, cfg, args, PREFILL_TOKENS, repeats=5, seed=2)
         print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
                                       "ms": round(1e3 * seconds, 3)}}))
         return 0
 
-    elapsed, mean_context = decode_run(runner, cfg, args.batch, steps, args.warmup, seed=1, prompt_len=prompt_len)
+    serving = Serving(runner, cfg, args, args.batch, prompt_len, args.steps + args.warmup + (24 if args.mixed else 0),
+                      seed=1, room=1 if args.mixed else 0)
+    steps = min(args.steps, serving.ticks - args.warmup - (24 if args.mixed else 0))
+    elapsed, mean_context = serving.timed_ticks(steps, args.warmup)
+    mixed_ms = serving.mixed_tick_ms(repeats=5) if args.mixed else None
+    serving.finish()
     ms_per_step = 1e3 * elapsed / steps
     value = args.batch * steps / elapsed
-    per_token = runner.manager.bytes_per_token
-    step_bytes = weight_bytes(runner) + mean_context * per_token
+    step_bytes = weight_bytes(runner) + mean_context * runner.manager.bytes_per_token
     achieved = step_bytes / (elapsed / steps)
 
     headline = (args.shape == "4b" and args.batch == 8 and prompt_len == PROMPT_LEN and args.dtype == "bfloat16"
@@ -359,17 +355,20 @@ def main() -> int:
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
             "global_batch": args.batch, "seq_len": prompt_len, "new_tokens": steps,
             "context_length": context_length, "page_size": PAGE_SIZE, "prefill_tokens": PREFILL_TOKENS,
-            "hip_graphs": runner.graphs is not None, "parallelism": "single-gpu",
+            "hip_graphs": runner.graphs is not None, "pool_pages": runner.manager.num_pages,
+            "startup_s": round(runner.startup["total_s"], 2), "parallelism": "single-gpu",
             "baseline": "reference on one NVIDIA L4, 8 clients: 199.8 tokens/s",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_BYTES_PER_S / 1e9,
                      "unit": "GB/s", "frac": round(achieved / HBM_BYTES_PER_S, 4)},
+        "startup": {k: round(v, 2) for k, v in runner.startup.items()},
     }
+    if runner.graphs is not None:
+        record["startup"]["graphs"] = len(runner.graphs.captured)
     if not args.no_prefill:
-        seconds = prefill_run(runner, cfg, repeats=5, seed=2)
-        attention = 4.0 * cfg.num_hidden_layers * cfg.num_attention_heads * cfg.head_dim * (
-            PREFILL_TOKENS * (PREFILL_TOKENS + 1) / 2)
-        flops = linear_flops_per_token(cfg) * PREFILL_TOKENS + attention + 2.0 * cfg.hidden_size * cfg.vocab_size
+        seconds = prefill_run(runner, cfg, args, PREFILL_TOKENS, repeats=5, seed=2)
+        flops = (linear_flops_per_token(cfg) * PREFILL_TOKENS + attention_flops(cfg, PREFILL_TOKENS)
+                 + 2.0 * cfg.hidden_size * cfg.vocab_size)
         record["prefill"] = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
                              "ms": round(1e3 * seconds, 3),
                              "frac": round(flops / seconds / PEAK_FLOPS[dtype_key], 4)}
@@ -380,20 +379,41 @@ def main() -> int:
         if "prefill" in record and dtype_key == "bf16":
             record["prefill"]["frac_of_measured"] = round(
                 record["prefill"]["frac"] * PEAK_FLOPS[dtype_key] / 1e12 / peaks["bf16_gemm_tflops"], 4)
-    if args.mixed:
-        seconds = mixed_run(runner, cfg, args.batch, prompt_len, repeats=5, seed=4)
-        record["mixed"] = {"decodes": args.batch, "chunk": PREFILL_TOKENS, "ms": round(1e3 * seconds, 3)}
+    if mixed_ms is not None:
+        record["mixed"] = {"decodes": args.batch, "chunk": PREFILL_TOKENS, "ms": round(mixed_ms, 3)}
     if not args.no_points:
         points = {}
-        for batch in (1, 64):
-            n = min(steps, 256)
-            e, _ = decode_run(runner, cfg, batch, n, args.warmup, seed=3 + batch, prompt_len=prompt_len)
-            points[f"decode_b{batch}"] = round(batch * n / e, 1)
-        rate, first_ms = engine_run(runner, cfg, batch=8, seed=9, prompt_len=prompt_len)
+        few = max(32, min(steps, 256))
+
+        def put(name, point):
+            points[name] = round(point["tokens_per_s"], 1)
+            points[name + "_hbm_frac"] = round(point["frac"], 4)
+
+        put("decode_b1", decode_point(runner, cfg, args, 1, prompt_len, few, seed=4))
+        put("decode_b64", decode_point(runner, cfg, args, 64, prompt_len, few, seed=67))
+        if headline:
+            # longer contexts: the decode attention's share grows, its keys are cut over workgroups
+            put("decode_b8_ctx4096", decode_point(runner, cfg, args, 8, 4096, 64, seed=11))
+            put("decode_b1_ctx8000", decode_point(runner, cfg, args, 1, 8000, 64, seed=12))
+            point = decode_point(runner, cfg, args, 64, 4096, 64, seed=13, mixed=True)
+            put("decode_b64_ctx4096", point)
+            # a step of 64 decoded tokens (about 4,200 cached each) beside a 2,048-token portion
+            chunk_flops = (linear_flops_per_token(cfg) * (PREFILL_TOKENS + 64) + attention_flops(cfg, PREFILL_TOKENS)
+                           + 65 * 2.0 * cfg.hidden_size * cfg.vocab_size)
+            points["mixed_b64_chunk2048_ms"] = round(point["mixed_ms"], 3)
+            points["mixed_b64_chunk2048_hbm_frac"] = round(point["bytes"] / (point["mixed_ms"] * 1e-3) / HBM_BYTES_PER_S, 4)
+            points["mixed_b64_chunk2048_flops_frac"] = round(chunk_flops / (point["mixed_ms"] * 1e-3) / PEAK_FLOPS[dtype_key], 4)
+            # one prompt of 8,191 tokens (the context's 8,192 less the token it produces), four portions
+            long_prompt = context_length - 1
+            seconds = prefill_run(runner, cfg, args, long_prompt, repeats=3, seed=14)
+            flops = linear_flops_per_token(cfg) * long_prompt + attention_flops(cfg, long_prompt)
+            points["prefill_8191"] = round(long_prompt / seconds, 1)
+            points["prefill_8191_flops_frac"] = round(flops / seconds / PEAK_FLOPS[dtype_key], 4)
+        rate, first_ms = engine_run(runner, cfg, args, batch=8, seed=9, prompt_len=prompt_len)
         points["engine_b8"], points["engine_b8_first_token_ms"] = round(rate, 1), round(first_ms, 2)
         # the reference's other published workload: 2,048-token prompts, 32 new tokens, 8 at a time
         # (53.7 output tokens/s and 847 ms to the first token on its L4, /root/reference/README.md:76,90)
-        rate, first_ms = engine_run(runner, cfg, batch=8, seed=10, prompt_len=PREFILL_TOKENS, new_tokens=32)
+        rate, first_ms = engine_run(runner, cfg, args, batch=8, seed=10, prompt_len=PREFILL_TOKENS, new_tokens=32)
         points["engine_prefill_heavy_b8"] = round(rate, 1)
         points["engine_prefill_heavy_b8_first_token_ms"] = round(first_ms, 2)
         record["points"] = points

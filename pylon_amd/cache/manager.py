@@ -39,6 +39,65 @@ def bytes_per_token(requirements: Seq[object], dtype: torch.dtype) -> int:
     return sum(2 * r.n_kv_heads * r.head_dim * elem for r in requirements if isinstance(r, KVRequirement))
 
 
+def group_requirements(requirements: Seq[object]):
+    """Runs by what they keep: ``({KVRequirement: [run ids]}`` in order of first appearance,
+    one entry per group of pages; ``{run id: StateRequirement})``."""
+    by_need: Dict[KVRequirement, List[int]] = {}
+    states: Dict[int, StateRequirement] = {}
+    for cache_id, need in enumerate(requirements):
+        if need is None:
+            continue
+        if isinstance(need, KVRequirement):
+            by_need.setdefault(need, []).append(cache_id)
+        elif isinstance(need, StateRequirement):
+            states[cache_id] = need
+        else:
+            raise TypeError(f"run {cache_id} asks for an unknown kind of cache: {need!r}")
+    return by_need, states
+
+
+def plan_pool(budget_bytes: int, groups: Seq[object], *, page_size: int, max_requests: int,
+              max_positions: Optional[int], chunk: int) -> List[int]:
+    """Pages for each group of runs under a budget of bytes.  ``groups[g]`` has
+    ``bytes_per_token`` (over the group's runs) and ``window``.
+
+    Every group has to hold the same requests, so every group gets the same number of pages P,
+    the largest the budget pays for, except that no group gets more than it can ever use: a
+    group that keeps every token, ``max_requests`` requests of ``max_positions`` tokens; a group
+    with a window, per request the pages of ``window + chunk`` tokens and one more (a step
+    takes the pages of up to ``chunk`` new tokens before it gives back those the window has
+    passed).  The reference's single group gets ``budget // bytes of a page``
+    (/root/reference/src/pylon/engine.py:173-178), capped as above."""
+    if not groups:
+        return []
+    full = pages_for(max_positions, page_size) * max_requests if max_positions else None
+    caps: List[Optional[int]] = []
+    for group in groups:
+        cap = full
+        if group.window is not None:
+            own = (pages_for(group.window + chunk, page_size) + 1) * max_requests
+            cap = own if cap is None else min(cap, own)
+        caps.append(cap)
+
+    def cost(pages: int) -> int:
+        return sum((pages if cap is None else min(pages, cap)) * page_size * group.bytes_per_token
+                   for group, cap in zip(groups, caps))
+
+    high = max(budget_bytes, 0) // max(1, page_size * min(g.bytes_per_token for g in groups)) + 1
+    if all(cap is not None for cap in caps):
+        high = min(high, max(caps))
+    low = 0  # the largest P known to fit
+    while low < high:
+        mid = (low + high + 1) // 2
+        if cost(mid) <= budget_bytes:
+            low = mid
+        else:
+            high = mid - 1
+    if low < 1:
+        raise RuntimeError("Not enough GPU memory remains for the KV cache and activations.")
+    return [low if cap is None else min(low, cap) for cap in caps]
+
+
 class KVGroup:
     """Runs with one key/value geometry: a pool of page ids and one K and V tensor per run."""
 
@@ -106,33 +165,35 @@ class CacheView:
 
 
 class CacheManager:
-    def __init__(self, requirements: Seq[object], *, page_size: int, num_pages: int, max_requests: int,
+    def __init__(self, requirements: Seq[object], *, page_size: int, num_pages, max_requests: int,
                  dtype: torch.dtype, device="cpu") -> None:
         """``requirements[c]`` is what run ``c`` of the schedule needs: a
         :class:`KVRequirement`, a :class:`StateRequirement`, or None (it borrows, or keeps
-        nothing).  Every group gets ``num_pages`` pages of ``page_size`` tokens."""
+        nothing).  ``num_pages``: pages (of ``page_size`` tokens) of every group, or one
+        number per group in the order of :func:`group_requirements`."""
         if page_size < 1:
             raise ValueError("page_size must be positive")
         self.page_size = page_size
-        self.num_pages = num_pages
         self.dtype = dtype
         self.device = device
         self.n_caches = len(requirements)
         self.groups: List[KVGroup] = []
         self.group_of: Dict[int, int] = {}
         self.slots = StateSlots(max_requests)
-        by_need: Dict[KVRequirement, List[int]] = {}
-        for cache_id, need in enumerate(requirements):
-            if need is None:
-                continue
-            if isinstance(need, KVRequirement):
-                by_need.setdefault(need, []).append(cache_id)
-            elif isinstance(need, StateRequirement):
-                self.slots.add_state(cache_id, tuple(need.shape), need.dtype, device)
-            else:
-                raise TypeError(f"run {cache_id} asks for an unknown kind of cache: {need!r}")
-        for need, cache_ids in by_need.items():
-            group = KVGroup(len(self.groups), need, cache_ids, num_pages, page_size, dtype, device,
+        by_need, states = group_requirements(requirements)
+        for cache_id, need in states.items():
+            self.slots.add_state(cache_id, tuple(need.shape), need.dtype, device)
+        if isinstance(num_pages, int):
+            per_group = [num_pages] * len(by_need)
+        else:
+            per_group = [int(n) for n in num_pages]
+            if len(per_group) != len(by_need):
+                raise ValueError(f"{len(per_group)} page counts for {len(by_need)} groups of runs")
+        # What admission counts with: the pages of the group that has most (one that keeps
+        # every token, if there is one; a group with a window may have fewer and never lacks).
+        self.num_pages = max(per_group) if per_group else (num_pages if isinstance(num_pages, int) else 0)
+        for (need, cache_ids), pages in zip(by_need.items(), per_group):
+            group = KVGroup(len(self.groups), need, cache_ids, pages, page_size, dtype, device,
                             max_requests)
             self.groups.append(group)
             for cache_id in cache_ids:
@@ -260,6 +321,23 @@ class CacheManager:
         seq.closed = True
         seq._pending = None
         self._live.pop(seq.request_id, None)
+
+    # ---- fixed-size state across a step that may fail ---------------------------------
+    def snapshot_state(self, seqs: Seq[Sequence]):
+        """A copy of the fixed-size state of these requests, to put back should the step
+        fail after a mixer has overwritten it.  None when no run keeps such state (then
+        nothing is copied: the case of every model of keys and values only)."""
+        if not self.slots.tensors:
+            return None
+        index = torch.as_tensor([seq.slot for seq in seqs], dtype=torch.long, device=self.device)
+        return index, {cache_id: tensor.index_select(0, index) for cache_id, tensor in self.slots.tensors.items()}
+
+    def restore_state(self, saved) -> None:
+        if saved is None:
+            return
+        index, copies = saved
+        for cache_id, copy in copies.items():
+            self.slots.tensors[cache_id].index_copy_(0, index, copy)
 
     # ---- what a step needs to know ---------------------------------------------------
     def table_width(self, seqs: Seq[Sequence], counts: Seq[int]) -> int:

@@ -66,6 +66,10 @@ OPTIONS = (
     Option("max_queue_size", 32, int, lambda v: _whole(v) and v >= 1, "a whole number of at least 1"),
     Option("batch_wait_ms", 2.0, float, lambda v: _real(v) and v >= 0, "a finite number of at least 0"),
     Option("cuda_graphs", False, _flag, lambda v: isinstance(v, bool), "true or false"),
+    # Start-up captures the decode graphs of requests of up to this many tokens (unset: of the
+    # longest request the model and the pool allow); graphs of longer ones at their first use.
+    Option("cuda_graph_max_tokens", None, _optional_int, lambda v: v is None or (_whole(v) and v >= 1),
+           "a whole number of at least 1, or unset"),
     Option("admit_skip", 4, int, lambda v: _whole(v) and v >= 0, "a whole number of at least 0"),
     Option("page_size", 256, int, lambda v: _whole(v) and v >= 16 and v % 16 == 0, "a positive multiple of 16"),
     # Queue the next step before the host has read the tokens of the running one (they are
@@ -90,6 +94,7 @@ class PylonConfig:
     max_queue_size: int = _BY_NAME["max_queue_size"].default
     batch_wait_ms: float = _BY_NAME["batch_wait_ms"].default
     cuda_graphs: bool = _BY_NAME["cuda_graphs"].default
+    cuda_graph_max_tokens: Optional[int] = _BY_NAME["cuda_graph_max_tokens"].default
     admit_skip: int = _BY_NAME["admit_skip"].default
     page_size: int = _BY_NAME["page_size"].default
     run_ahead: bool = _BY_NAME["run_ahead"].default

@@ -71,6 +71,16 @@ class MetadataArena:
             event.synchronize()
         return self._host[index].numpy(), index
 
+    def stage(self, values: np.ndarray) -> torch.Tensor:
+        """A new int32 device tensor holding ``values``, copied through one of the pinned
+        buffers without making the host wait for the device."""
+        flat = np.ascontiguousarray(values, dtype=np.int32).reshape(-1)
+        host, index = self.acquire(flat.size)
+        host[: flat.size] = flat
+        out = torch.empty(flat.size, dtype=torch.int32, device=self.device)
+        self.upload(index, flat.size, into=out)
+        return out.view(values.shape)
+
     def upload(self, index: int, size: int, into: Optional[torch.Tensor] = None) -> torch.Tensor:
         target = self._device_buf if into is None else into
         target[:size].copy_(self._host[index][:size], non_blocking=True)
@@ -107,6 +117,7 @@ class StepContext:
     logit_slots: Optional[torch.Tensor] = None  # int32 [n]: state slot of each wanted row's request
     chosen: Optional[torch.Tensor] = None  # int32 [slots]: last sampled token per state slot
     logits_out: Optional[torch.Tensor] = None  # float32 [>= n_logits, vocab]: where the logits go, if given
+    arena: Optional[MetadataArena] = None  # pinned staging for what parts put on the device themselves
     _tiles: Dict[Tuple[int, int], torch.Tensor] = field(default_factory=dict)
 
     def cache(self, cache_id: int) -> CacheView:
@@ -138,8 +149,11 @@ class StepContext:
             np.cumsum(self.counts, out=starts[1:])
             table = np.stack([starts[row] + within, count, row, self.starts[row] + within], axis=1)
             order = np.argsort(-(table[:, 3] + table[:, 1]), kind="stable")
-            host = torch.from_numpy(np.ascontiguousarray(table[order].astype(np.int32)))
-            tiles = host.to(self.token_ids.device)
+            ordered = table[order].astype(np.int32)
+            if self.arena is not None:
+                tiles = self.arena.stage(ordered)
+            else:
+                tiles = torch.from_numpy(np.ascontiguousarray(ordered)).to(self.token_ids.device)
             self._tiles[key] = tiles
         return tiles
 
@@ -264,7 +278,7 @@ def build_step(entries: Seq[StepEntry], manager: CacheManager, arena: MetadataAr
             views=views, counts=counts, starts=starts, max_count=int(counts.max()),
             max_len=int(seq_lens.max()) if len_bound is None else int(len_bound),
             decode_only=bool((counts == 1).all()),
-            fixed_shapes=fixed_shapes,
+            fixed_shapes=fixed_shapes, arena=arena,
         )
     except BaseException:
         manager.cancel(pairs)

@@ -183,19 +183,21 @@ class Engine:
         return cls(PylonConfig(model_path=str(folder), **options), threaded=threaded)
 
     @classmethod
-    def from_random(cls, model_config: dict, seed: int = 0, *, std: float = 0.02, norm_jitter: float = 0.0,
+    def from_random(cls, model_config: dict, seed: int = 0, *, std: Optional[float] = None,
+                    norm_jitter: float = 0.0, draw_on=None, config: Optional[PylonConfig] = None,
                     **options) -> "Engine":
         """An engine over random weights of the architecture and sizes that ``model_config``
-        (the contents of a config.json) names: the folder that the random-weights mode
-        writes from (config, seed), loaded like any other and then deleted."""
-        import tempfile
+        (the contents of a config.json) names, drawn in place on the device by the
+        random-weights mode's rule (``draw_on="cpu"``: the very numbers of the folder that the
+        mode writes from the same config and seed).  Serving options as ``config`` or as
+        keywords.  Start-up is :meth:`Runner.from_random`: the same fit check, pool sizing and
+        graph capture as for a model folder."""
+        from .runner import Runner
 
-        from ..weights import write_random_model
-
-        with tempfile.TemporaryDirectory(prefix="pylon_random_") as tmp:
-            folder = write_random_model(tmp, model_config, seed, dtype=options.get("dtype", "bfloat16"),
-                                        std=std, norm_jitter=norm_jitter)
-            return cls.from_folder(folder, **options)
+        threaded = options.pop("threaded", False)
+        config = config if config is not None else PylonConfig(**options)
+        runner = Runner.from_random(model_config, seed, config, std=std, norm_jitter=norm_jitter, draw_on=draw_on)
+        return cls(config, runner=runner, threaded=threaded)
 
     # ---- the public surface -------------------------------------------------------------
     def enqueue(self, input_ids: Sequence[int], eos_token_id=None, sampling: Optional[Sampling] = None,
@@ -290,10 +292,13 @@ class Engine:
     def tick(self) -> bool:
         """One round of admit, step, sample, finish.  True while work remains.
 
-        The engine's lock guards its queue and its lists of requests, not the device: the one
-        place where a tick waits for the device, reading a step's sampled tokens, happens
-        with the lock released, so that ``enqueue``, ``snapshot`` and ``close`` from other
-        threads never wait for a step.  Ticks themselves run one at a time."""
+        The engine's lock guards its queue and its lists of requests, not the device: where a
+        tick waits for the device (reading a step's sampled tokens, or the end of a step that
+        sampled nothing), it has released the lock, so that ``enqueue``, ``snapshot`` and
+        ``close`` from other threads do not wait for a step.  One exception: a decode graph
+        that start-up did not capture (a request longer than ``cuda_graph_max_tokens``) is
+        captured at its first use, inside the step, under the lock.  Ticks themselves run one
+        at a time."""
         with self._ticking:
             with self._lock:
                 if self._closed:
@@ -430,7 +435,7 @@ class Engine:
             for item in ready:
                 item.unread += 1
         elif not self._run_ahead and hasattr(self.runner, "synchronize"):
-            self.runner.synchronize()
+            draw = _Finished(self.runner)  # nothing sampled: tick waits for the step, lock released
         return Flight(draw, ready, decoding, portions, started)
 
     def _land(self, flight: Flight, token_ids: Sequence[int]) -> None:
@@ -552,6 +557,17 @@ class Engine:
             except Exception as error:  # noqa: BLE001 - a broken tick fails what runs
                 with self._lock:
                     self._fail_active(error)
+
+
+class _Finished:
+    """A step that sampled nothing: waiting for it yields no token ids."""
+
+    def __init__(self, runner) -> None:
+        self._runner = runner
+
+    def result(self) -> List[int]:
+        self._runner.synchronize()
+        return []
 
 
 class _Drawn:

@@ -9,10 +9,12 @@ captured at start-up (``Runner.capture_graphs``) is captured the first time its 
 is seen, and a batch is never padded to a larger captured size.
 
 The launches recorded in a graph must not depend on the requests' lengths: the block
-table has a fixed width, and how the decode attention kernel shares a request's keys
-between workgroups and waves depends on the batch size and on a bound on the lengths
-only.  That bound is a power of two of at least 1024 tokens; there is one graph per
-(batch size, bound).
+table has a fixed width, and what a mixer launches may depend on the batch size and on a
+bound on the lengths only (the decode attention kernel shares a request's keys between
+workgroups and waves by it).  That bound is a power of two of at least 1024 tokens.  A
+mixer says through ``decode_signature(rows, bound)`` what of its launches depends on the
+bound; bounds with equal signatures share one graph, and a mixer that does not say is taken
+to depend on the bound itself.  There is one graph per (batch size, signature).
 """
 from __future__ import annotations
 
@@ -49,7 +51,13 @@ class DecodeGraphs:
         self.replays = 0
 
     def captured_sizes(self):
-        return tuple(sorted({rows for rows, _bound in self.captured}))
+        return tuple(sorted({rows for rows, _signature in self.captured}))
+
+    def key(self, rows: int, bound: int) -> tuple:
+        """What names the graph of ``rows`` requests of at most ``bound`` tokens: the batch
+        size and everything the model's recorded launches take from the bound."""
+        describe = getattr(self.model, "decode_signature", None)
+        return rows, (("bound", bound) if describe is None else describe(rows, bound))
 
     def _bound(self, entries: Seq[StepEntry]) -> int:
         """The power of two (from 1024) that holds the longest request after this step."""
@@ -71,7 +79,7 @@ class DecodeGraphs:
     def wants(self, entries: Seq[StepEntry]) -> bool:
         """A decode-only step: one token per request, each wanting its logits."""
         rows = len(entries)
-        if rows > self.max_batch or (rows, self._bound(entries)) in self.failed:
+        if rows > self.max_batch or self.key(rows, self._bound(entries)) in self.failed:
             return False
         page = self.manager.page_size
         for e in entries:
@@ -91,7 +99,7 @@ class DecodeGraphs:
         manager, model, arena = self.manager, self.model, self.arena
         pairs = [(e.seq, 1) for e in entries]
         bound = max(bound or 0, self._bound(entries))
-        key = (rows, bound)
+        key = self.key(rows, bound)
         entry = self.captured.get(key)
         if entry is None:
             _, size = plan_layout(rows, rows, rows, len(manager.groups), self.width)

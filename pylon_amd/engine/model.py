@@ -62,6 +62,19 @@ class Model(Part):
                     )
         return needs
 
+    def decode_signature(self, rows: int, bound: int) -> tuple:
+        """What the launches of a decode-only step of ``rows`` requests take from a bound on
+        the requests' lengths, over all layers: two bounds with equal signatures record the
+        same graph.  A block or mixer without ``decode_signature`` is taken to depend on the
+        bound itself."""
+        seen = []
+        for block in self.blocks:
+            describe = getattr(block, "decode_signature", None)
+            signature = ("bound", bound) if describe is None else describe(rows, bound)
+            if signature not in seen:
+                seen.append(signature)
+        return tuple(seen)
+
     @property
     def head_weight(self) -> torch.Tensor:
         return self.params["embed"] if self.spec.tie_word_embeddings else self.params["lm_head"]

@@ -610,6 +610,21 @@ def _ids_out(rows: int, device, out: Optional[torch.Tensor]) -> torch.Tensor:
     return out
 
 
+_argmax_scratch: dict = {}
+
+
+def _argmax_partials(rows: int, device: torch.device) -> torch.Tensor:
+    """The first launch leaves up to 64 partial results of 8 bytes per row for the second: one
+    buffer per device, kept and grown, so that a serving loop allocates nothing per step.
+    Calls on one stream follow each other; callers on other streams bring their own order."""
+    need = max(rows, 1) * 64 * 8
+    have = _argmax_scratch.get(device)
+    if have is None or have.numel() < need:
+        have = torch.empty((max(need, 256 * 64 * 8),), dtype=torch.uint8, device=device)
+        _argmax_scratch[device] = have
+    return have
+
+
 def argmax(logits: torch.Tensor, *, out: Optional[torch.Tensor] = None,
            chosen: Optional[torch.Tensor] = None, place: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The index of each row's largest logit (the lowest among equals); with ``chosen`` and
@@ -621,8 +636,7 @@ def argmax(logits: torch.Tensor, *, out: Optional[torch.Tensor] = None,
         raise KernelError("argmax takes float32 logits on the GPU")
     out = _ids_out(rows, logits.device, out)
     chosen_ptr, place_ptr = _chosen_args(rows, chosen, place)
-    # the first launch leaves up to 64 partial results of 8 bytes per row for the second
-    scratch = torch.empty((max(rows, 1) * 64 * 8,), dtype=torch.uint8, device=logits.device)
+    scratch = _argmax_partials(rows, logits.device)
     _lib.call("pylon_argmax", out.data_ptr(), logits.data_ptr(), rows, vocab, logits.stride(0),
               chosen_ptr, place_ptr, scratch.data_ptr(), scratch.numel(), _stream())
     return out

@@ -34,6 +34,8 @@ def _add_serving_options(p: argparse.ArgumentParser) -> None:
     p.add_argument("--num-pages", type=int)
     p.add_argument("--cuda-graphs", action="store_true", default=None,
                    help="replay decode-only steps from HIP graphs")
+    p.add_argument("--cuda-graph-max-tokens", type=int,
+                   help="capture at start-up the graphs of requests of up to this many tokens")
     p.add_argument("--no-run-ahead", dest="run_ahead", action="store_false", default=None,
                    help="read every step's tokens before the next step is queued")
 
@@ -59,7 +61,7 @@ def _generate(args) -> int:
         weight_headroom_ratio=args.weight_headroom_ratio,
         kv_cache_headroom_ratio=args.kv_cache_headroom_ratio, admit_skip=args.admit_skip,
         page_size=args.page_size, num_pages=args.num_pages, cuda_graphs=args.cuda_graphs,
-        run_ahead=args.run_ahead,
+        cuda_graph_max_tokens=args.cuda_graph_max_tokens, run_ahead=args.run_ahead,
     )
     prompts = [_parse_ids(text) for text in args.prompt_ids or []]
     if args.prompt_file:
@@ -73,10 +75,7 @@ def _generate(args) -> int:
         if args.model:
             print("give --model or --random, not both", file=sys.stderr)
             return 2
-        import dataclasses
-
-        options = {k: v for k, v in dataclasses.asdict(config).items() if k != "model_path"}
-        engine = Engine.from_random(json.loads(Path(args.random).read_text()), args.seed, **options)
+        engine = Engine.from_random(json.loads(Path(args.random).read_text()), args.seed, config=config)
     else:
         engine = Engine(config)
     try:

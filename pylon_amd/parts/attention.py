@@ -46,6 +46,12 @@ class Attention(Part):
         """The most keys a token of this step attends to."""
         return ctx.max_len if self.spec.window is None else min(ctx.max_len, self.spec.window)
 
+    def decode_signature(self, rows: int, bound: int) -> tuple:
+        """Of a bound on the lengths, a decode-only step's launches take only how the keys of
+        a request are shared between workgroups and waves."""
+        span = bound if self.spec.window is None else min(bound, self.spec.window)
+        return ("attention",) + tuple(ops.decode_launch(rows, self.spec.n_kv_heads, span))
+
     def forward(self, h: torch.Tensor, ctx, cache, stores: bool) -> torch.Tensor:
         spec = self.spec
         tokens = h.shape[0]

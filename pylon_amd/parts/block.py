@@ -33,6 +33,10 @@ class PreNormBlock(Part):
     def cache_requirement(self):
         return self.mixer.cache_requirement()
 
+    def decode_signature(self, rows: int, bound: int) -> tuple:
+        describe = getattr(self.mixer, "decode_signature", None)
+        return ("bound", bound) if describe is None else describe(rows, bound)
+
     def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], ctx, cache,
                 stores: bool) -> Tuple[torch.Tensor, torch.Tensor]:
         h = self.mixer_norm.add_forward(resid, delta)

@@ -33,7 +33,7 @@ def run(verbose: bool = True) -> None:
 
     prompt = np.random.default_rng(3).integers(0, TINY["vocab_size"], 21).tolist()
     with tempfile.TemporaryDirectory(prefix="pylon_selftest_") as tmp:
-        folder = write_random_model(tmp, TINY, seed=1, dtype="float32", std=0.08, norm_jitter=0.1)
+        folder = write_random_model(tmp + "/float32", TINY, seed=1, dtype="float32", std=0.08, norm_jitter=0.1)
         exact = Runner.from_folder(folder, dtype="float32", page_size=16, num_pages=8, max_requests=2)
         whole = exact.open("whole")
         want = exact.step([StepEntry(whole, prompt, list(range(len(prompt))))]).cpu()
@@ -51,7 +51,12 @@ def run(verbose: bool = True) -> None:
         exact.close(whole)
         exact.close(single)
 
-        half = Runner.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=8, max_requests=2)
+        # the same numbers stored in bfloat16: matrices stay bfloat16 and run on the matrix-core
+        # kernels (a folder stored in 32-bit would keep them in 32-bit and on the exact kernels)
+        rounded = write_random_model(tmp + "/bfloat16", TINY, seed=1, dtype="bfloat16", std=0.08, norm_jitter=0.1)
+        half = Runner.from_folder(rounded, dtype="bfloat16", page_size=16, num_pages=8, max_requests=2)
+        if half.model.params["embed"].dtype != torch.bfloat16:
+            raise AssertionError("a folder stored in bfloat16 was not loaded as bfloat16")
         seq = half.open("half")
         got = half.step([StepEntry(seq, prompt, list(range(len(prompt))))]).cpu()
         half.close(seq)

@@ -67,14 +67,13 @@ def _param_dtype(model_dtype: torch.dtype, role: str, stored: List[str]) -> torc
     return torch.bfloat16
 
 
-def load_weights(model, arch: Architecture, config, folder, *, strict: bool = False) -> List[str]:
-    """Fill ``model``'s parameters from ``folder``; raise :class:`WeightsError` listing
-    every missing, wrongly shaped and unexpected tensor if a needed tensor is missing or
-    wrong (with ``strict``: also if only unexpected ones are found).  Returns the names of
-    the tensors that were skipped because the architecture does not know them."""
-    folder = Path(folder)
+def _scan(model, arch: Architecture, config, folder: Path, strict: bool):
+    """Read the shards' headers and hold them against what the architecture needs.  Returns
+    (targets, {tensor name: (file, shape, stored type)}, unexpected names); raises
+    :class:`WeightsError` listing every problem if a needed tensor is missing or wrong (with
+    ``strict``: also if only unexpected ones are found).  No tensor data is read."""
     targets: Dict[str, WeightTarget] = arch.weight_targets(config)
-    params = {path: (owner, name) for path, owner, name in model.named_params()}
+    params = {path for path, _owner, _name in model.named_params()}
     files = shard_files(folder)
     for path in files:
         if not path.is_file():
@@ -108,21 +107,57 @@ def load_weights(model, arch: Architecture, config, folder, *, strict: bool = Fa
     missing = [n for n, t in targets.items() if n not in present and not t.optional]
     if missing or wrong or (strict and unexpected):
         raise WeightsError(missing, unexpected, wrong)
+    return targets, found, unexpected
+
+
+def _decide_dtypes(model, targets, found) -> Dict[str, torch.dtype]:
+    """Each parameter's element type from what is stored for it."""
+    params = {path: (owner, name) for path, owner, name in model.named_params()}
+    stored_by_param: Dict[str, List[str]] = {}
+    for name, (_path, _shape, stored) in found.items():
+        stored_by_param.setdefault(targets[name].param, []).append(stored)
+    out = {}
+    for param_path, stored in stored_by_param.items():
+        owner, pname = params[param_path]
+        out[param_path] = _param_dtype(model.dtype, owner.param_roles[pname], stored)
+    return out
+
+
+def stored_param_dtypes(model, arch: Architecture, config, folder) -> Dict[str, torch.dtype]:
+    """``{parameter path: the element type it has once the folder is loaded}``, from the
+    shards' headers alone; ``model`` may live on the meta device.  What start-up counts the
+    weights' bytes with before anything is allocated: a matrix stored in 32-bit stays 32-bit
+    in a bfloat16 model and takes twice the bytes."""
+    targets, found, _unexpected = _scan(model, arch, config, Path(folder), strict=False)
+    return _decide_dtypes(model, targets, found)
+
+
+def load_weights(model, arch: Architecture, config, folder, *, strict: bool = False) -> List[str]:
+    """Fill ``model``'s parameters from ``folder``; raise :class:`WeightsError` listing
+    every missing, wrongly shaped and unexpected tensor if a needed tensor is missing or
+    wrong (with ``strict``: also if only unexpected ones are found).  Returns the names of
+    the tensors that were skipped because the architecture does not know them."""
+    folder = Path(folder)
+    targets, found, unexpected = _scan(model, arch, config, folder, strict)
+    params = {path: (owner, name) for path, owner, name in model.named_params()}
     if unexpected:
         logger.warning("weights_skipped folder=%s count=%d names=%s", folder, len(unexpected),
                        ", ".join(sorted(unexpected)[:8]) + (" ..." if len(unexpected) > 8 else ""))
 
-    # Decide each parameter's element type from what is stored for it, then copy.
-    stored_by_param: Dict[str, List[str]] = {}
-    for name, (_path, _shape, stored) in found.items():
-        stored_by_param.setdefault(targets[name].param, []).append(stored)
-    for param_path, stored in stored_by_param.items():
+    kept_wide = []
+    for param_path, want in _decide_dtypes(model, targets, found).items():
         owner, pname = params[param_path]
-        role = owner.param_roles[pname]
-        want = _param_dtype(model.dtype, role, stored)
         if owner.params[pname].dtype != want:
             old = owner.params[pname]
             owner.params[pname] = torch.empty(old.shape, dtype=want, device=old.device)
+        if want == torch.float32 and model.dtype != torch.float32 and owner.param_roles[pname] == "matrix":
+            kept_wide.append(param_path)
+    if kept_wide:
+        logger.warning(
+            "weights_kept_32bit folder=%s count=%d names=%s: matrices stored in 32-bit stay 32-bit in this "
+            "%s model; they take twice the memory and their products run on the exact float32 kernel",
+            folder, len(kept_wide), ", ".join(sorted(kept_wide)[:4]) + (" ..." if len(kept_wide) > 4 else ""),
+            str(model.dtype).replace("torch.", ""))
     filled: Dict[str, int] = {}
     by_file: Dict[Path, List[str]] = {}
     for name, (path, _shape, _stored) in found.items():

@@ -29,12 +29,15 @@ def _generator(seed: int, name: str, device="cpu") -> torch.Generator:
 _SLAB = 1 << 26  # elements drawn at a time, so that no float32 copy of a large matrix is needed
 
 
-def draw_tensor(seed: int, name: str, target, sigma: float, norm_jitter: float, *, out: torch.Tensor) -> None:
+def draw_tensor(seed: int, name: str, target, sigma: float, norm_jitter: float, *, out: torch.Tensor,
+                draw_on=None) -> None:
     """The one rule of the random-weights mode: fill ``out`` (of the target's shape, on any
     device, of any float type) with tensor ``name`` of seed ``seed``.  ``normal``:
     N(0, sigma^2); ``ones`` / ``ones_jitter``: 1, or 1 + norm_jitter * N(0, 1).  The numbers
-    come from a generator on ``out``'s device keyed by (seed, name): a folder written on the
-    CPU and a model filled on the GPU follow the same rule, but not the same numbers."""
+    come from a generator keyed by (seed, name) on the device ``draw_on`` (default: where
+    ``out`` lives): drawn on the CPU they are the numbers of the folder that
+    :func:`write_random_model` writes; drawn on a GPU they follow the same rule with other
+    numbers, a few hundred times faster."""
     if tuple(out.shape) != tuple(target.shape):
         raise ValueError(f"{name}: expected a tensor of shape {tuple(target.shape)}, got {tuple(out.shape)}")
     if target.init in ("ones", "ones_jitter") and not (target.init == "ones_jitter" and norm_jitter):
@@ -42,16 +45,17 @@ def draw_tensor(seed: int, name: str, target, sigma: float, norm_jitter: float, 
         return
     if target.init not in ("normal", "ones_jitter"):
         raise ValueError(f"unknown init rule {target.init!r} for {name}")
-    gen = _generator(seed, name, out.device)
+    where = torch.device(draw_on) if draw_on is not None else out.device
+    gen = _generator(seed, name, where)
     scale, shift = (sigma, 0.0) if target.init == "normal" else (norm_jitter, 1.0)
     if out.is_contiguous():
         flat = out.view(-1)
         for start in range(0, flat.numel(), _SLAB):
             part = flat[start: start + _SLAB]
-            part.copy_(torch.randn(part.numel(), generator=gen, dtype=torch.float32, device=out.device)
+            part.copy_(torch.randn(part.numel(), generator=gen, dtype=torch.float32, device=where)
                        * scale + shift)
     else:
-        out.copy_(torch.randn(tuple(out.shape), generator=gen, dtype=torch.float32, device=out.device)
+        out.copy_(torch.randn(tuple(out.shape), generator=gen, dtype=torch.float32, device=where)
                   * scale + shift)
 
 
@@ -89,11 +93,12 @@ def write_random_model(folder, config: Mapping, seed: int, *, dtype: str = "bflo
 
 
 def fill_random_model(model, arch, cfg, seed: int, *, std: Optional[float] = None,
-                      norm_jitter: float = 0.0) -> None:
-    """The same mode without the folder: fill ``model``'s parameters in place, on their
-    device, tensor by tensor through the architecture's table of checkpoint names (so fused
-    matrices get their parts in their row ranges, as a load would put them).  For models too
-    large to be worth writing to disk; every parameter must be covered."""
+                      norm_jitter: float = 0.0, draw_on=None) -> None:
+    """The same mode without the folder: fill ``model``'s parameters in place, tensor by
+    tensor through the architecture's table of checkpoint names (so fused matrices get their
+    parts in their row ranges, as a load would put them).  ``draw_on``: the device whose
+    generator draws (default: the parameters' own; ``"cpu"`` gives the folder's numbers).
+    Every parameter must be covered."""
     params = {path: (owner, name) for path, owner, name in model.named_params()}
     sigma = _sigma(cfg, std)
     covered = {path: 0 for path in params}
@@ -106,7 +111,7 @@ def fill_random_model(model, arch, cfg, seed: int, *, std: Optional[float] = Non
         dest = owner.params[pname]
         if dest.dim() >= 1 and len(target.shape) >= 1 and tuple(dest.shape) != tuple(target.shape):
             dest = dest[target.row_start: target.row_start + target.shape[0]]
-        draw_tensor(seed, name, target, sigma, norm_jitter, out=dest)
+        draw_tensor(seed, name, target, sigma, norm_jitter, out=dest, draw_on=draw_on)
         covered[target.param] += dest.numel()
     short = [path for path, (owner, pname) in params.items() if covered[path] != owner.params[pname].numel()]
     if short:

@@ -300,10 +300,62 @@ def test_a_replay_that_raises_leaves_the_cache_as_it_was():
     graphs.chosen, graphs.width, graphs.max_batch = None, 4, 4
     graphs.failed, graphs.replays, graphs.last_logit_slots = set(), 0, None
     block = torch.empty(256, dtype=torch.int32)
-    graphs.captured = {(1, 1024): (BrokenGraph(), block, None, None)}
+    graphs.captured = {graphs.key(1, 1024): (BrokenGraph(), block, None, None)}
     with pytest.raises(RuntimeError, match="replay failed"):
         graphs.run([StepEntry(a, [7], [0])])
     assert m.free_pages == free and a._pending is None and a.length == 4
     m.check()
     ctx = _ctx(m, [StepEntry(a, [7], [0])])
     assert ctx.positions.tolist() == [4]
+
+
+def test_a_budget_of_bytes_becomes_pages_per_group():
+    """Every group holds the same requests, so every group gets the same number of pages,
+    except that a group with a window never gets more than it can use; fixed-size state is
+    taken off the budget first (by the caller)."""
+    from types import SimpleNamespace as G
+
+    from pylon_amd.cache.manager import plan_pool
+
+    full, wide = G(bytes_per_token=100, window=None), G(bytes_per_token=300, window=None)
+    kw = dict(page_size=4, max_requests=2, max_positions=None, chunk=8)
+    # one group: the reference's budget // bytes of a page
+    assert plan_pool(10_000, [full], **kw) == [10_000 // 400]
+    # two groups that keep everything: one page of each costs 400 + 1200 bytes
+    assert plan_pool(16_000, [full, wide], **kw) == [10, 10]
+    assert plan_pool(15_999, [full, wide], **kw) == [9, 9]
+    # a position limit caps them: two requests of 20 tokens are ten pages
+    assert plan_pool(10 ** 9, [full, wide], page_size=4, max_requests=2, max_positions=20, chunk=8) == [10, 10]
+    # a window of 6 with portions of 8: per request pages_for(14) + 1 = 5 pages, so ten; what it
+    # does not need goes to the group beside it: 10 * 1200 + P * 400 <= 20,000 -> P = 20
+    window = G(bytes_per_token=300, window=6)
+    assert plan_pool(20_000, [full, window], **kw) == [20, 10]
+    assert plan_pool(8_000, [full, window], **kw) == [5, 5]  # below the window's cap both get P
+    with pytest.raises(RuntimeError, match="Not enough GPU memory"):
+        plan_pool(1_599, [full, wide], **kw)
+    assert plan_pool(123, [], **kw) == []
+    # the manager takes one count per group, and admission counts with the largest
+    m = CacheManager((FULL, KVRequirement(1, 16, window=6)), page_size=4, num_pages=[20, 10], max_requests=2,
+                     dtype=torch.float32)
+    assert [g.pool.num_pages for g in m.groups] == [20, 10] and m.num_pages == 20
+    assert m.groups[1].k[1].shape[0] == 10
+    with pytest.raises(ValueError, match="page counts"):
+        CacheManager((FULL,), page_size=4, num_pages=[20, 10], max_requests=2, dtype=torch.float32)
+
+
+def test_fixed_size_state_is_put_back_after_a_failed_step():
+    m = make(requirements=(FULL, StateRequirement((3,), torch.float32)), max_requests=3)
+    a, b, c = m.open("a"), m.open("b"), m.open("c")
+    state = m.view(1).state
+    state[a.slot], state[b.slot], state[c.slot] = 1.0, 2.0, 3.0
+    saved = m.snapshot_state([c, a])
+    state[a.slot] += 10.0  # what a mixer does before a later layer fails
+    state[c.slot] += 10.0
+    state[b.slot] += 10.0  # not part of the step: not put back
+    m.restore_state(saved)
+    assert state[a.slot].tolist() == [1.0] * 3 and state[c.slot].tolist() == [3.0] * 3
+    assert state[b.slot].tolist() == [12.0] * 3
+    # a model of keys and values only copies nothing
+    plain_manager = make()
+    assert plain_manager.snapshot_state([plain_manager.open("x")]) is None
+    plain_manager.restore_state(None)

@@ -202,3 +202,10 @@ def test_pool_pages_follow_the_reference_budget():
 
     with pytest.raises(RuntimeError, match="Not enough GPU memory"):
         pool_pages(free, total, 100_000, config, None)
+    # the measured branch (:85-95): the headroom is the activations' peak times 1 + ratio
+    from pylon_amd.engine.runner import cache_budget
+
+    assert cache_budget(free, total, config, activation_bytes=40_000) == 900_000 - 400_000 - 50_000
+    assert pool_pages(free, total, 100, config, None, activation_bytes=40_000) == 450_000 // 1600
+    with pytest.raises(ValueError, match="non-negative"):
+        cache_budget(free, total, config, activation_bytes=-1)

@@ -222,8 +222,9 @@ def test_running_ahead_gives_the_tokens_of_the_tick_by_tick_engine(tmp, graphs):
 
 
 def test_random_weights_straight_into_an_engine_and_the_command_line(tmp, tmp_path):
-    """Engine.from_random(config, seed) is the engine over the folder that the random-weights
-    mode writes from the same (config, seed); `main.py generate --random` prints its tokens."""
+    """Engine.from_random(config, seed, draw_on="cpu") is the engine over the folder that the
+    random-weights mode writes from the same (config, seed); drawn on the GPU (the default) the
+    numbers are others, the same on every run; `main.py generate --random` prints its tokens."""
     import json
     import subprocess
     import sys
@@ -238,7 +239,7 @@ def test_random_weights_straight_into_an_engine_and_the_command_line(tmp, tmp_pa
     sampling = Sampling(max_new_tokens=10, temperature=0.0)
     outputs = []
     for make in (lambda: Engine.from_folder(folder, dtype="bfloat16", page_size=64, num_pages=4),
-                 lambda: Engine.from_random(CONFIGS["D"], SEEDS["D"], norm_jitter=NORM_JITTER["D"],
+                 lambda: Engine.from_random(CONFIGS["D"], SEEDS["D"], norm_jitter=NORM_JITTER["D"], draw_on="cpu",
                                             dtype="bfloat16", page_size=64, num_pages=4)):
         engine = make()
         try:

@@ -118,7 +118,8 @@ def test_long_requests_share_their_keys_between_workgroups_in_graphs_too(tmp_pat
 
     eager_runner, eager = run(False)
     graph_runner, graphed = run(True)
-    assert {bound for _rows, bound in graph_runner.graphs.captured} == {2048, 4096}
+    graphs = graph_runner.graphs
+    assert set(graphs.captured) == {graphs.key(2, 2048), graphs.key(2, 4096)} and len(graphs.captured) == 2
     for rid in prompts:
         toks = prompts[rid] + decode[rid][:39]
         want = plain.forward(weights, cfg, toks)[len(prompts[rid]) - 1:]
@@ -159,15 +160,16 @@ def test_graphs_captured_at_start_up(tmp_path):
     assert small.capture_graphs() == (1, 2, 3)
     small.manager.check()
     assert small.manager.free_pages == 3
-    # by default only the smallest bound on the lengths is captured at start-up; on request
-    # every bound is, by short requests, and a long request then only replays
+    # up to a given length only the graphs of the bounds that hold it are captured; by default
+    # those of every bound are, by short requests, and a long request then only replays
     big = Runner.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=140, max_requests=3)
     big.enable_graphs(2)
     assert big.graphs.bounds() == (1024, 2048, 4096)
+    big.capture_graphs(max_tokens=1000)
+    assert set(big.graphs.captured) == {big.graphs.key(1, 1024), big.graphs.key(2, 1024)}
     big.capture_graphs()
-    assert set(big.graphs.captured) == {(1, 1024), (2, 1024)}
-    big.capture_graphs(bounds=big.graphs.bounds())
-    assert set(big.graphs.captured) == {(rows, bound) for rows in (1, 2) for bound in (1024, 2048, 4096)}
+    assert set(big.graphs.captured) == {big.graphs.key(rows, bound) for rows in (1, 2) for bound in (1024, 2048, 4096)}
+    assert len(big.graphs.captured) == 6  # two key/value heads: every bound cuts the keys otherwise
     plain_runner = Runner.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=140, max_requests=3)
     long_prompt = random_tokens(cfg["vocab_size"], 1100, 5)
     outs = []

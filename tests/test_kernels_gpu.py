@@ -707,7 +707,7 @@ def test_sampling_at_a_full_vocabulary_and_odd_layouts(ops):
 
 def test_sampling_with_thousands_of_equal_logits_at_the_boundary(ops):
     """More tokens in the top-p boundary's bin than the kernel gathers in LDS, most of them
-    equal: the kept set is still the rule's (a tie is kept or dropped as a whole)."""
+    equal: the kept set is the plain rule's, made whole where that rule cuts into a tie."""
     from tests.plain import qwen3 as plain
 
     vocab = 20000
@@ -726,11 +726,14 @@ def test_sampling_with_thousands_of_equal_logits_at_the_boundary(ops):
         first = ops.sample(dev, temps.to(DEV), tops.to(DEV), torch.zeros(3, device=DEV)).cpu().tolist()
         for r in range(3):
             row = f64(logits)[r]
-            p = np.exp(row - row.max())
-            p /= p.sum()
-            above = np.array([p[row > x].sum() for x in np.unique(row)])
-            keep_values = np.unique(row)[above <= top_p + 1e-12]
-            kept = np.nonzero(np.isin(row, keep_values) & (p * 2.0 ** 40 / p.max() >= 1))[0]
+            # The plain rule sorts and cuts wherever the cumulative mass passes top_p, inside a
+            # tie too (which of the equal tokens it keeps is an accident of its sort).  The
+            # kernel keeps every token at least as large as the smallest one the plain rule
+            # keeps: the same set, plus the rest of a tie the plain rule cut into.
+            p = plain.sampling_distribution(row, 1.0, top_p)
+            smallest_kept = row[p > 0].min()
+            mass = np.exp(row - row.max())
+            kept = np.nonzero((row >= smallest_kept) & (mass * 2.0 ** 40 >= 1))[0]
             assert first[r] == int(kept[0]) and last[r] == int(kept[-1]), (top_p, r, first[r], last[r])
     us = torch.tensor([0.3, 0.6, 0.9])
     _check_draws(ops, logits[1:2].repeat(3, 1), temps, torch.full((3,), 0.7), us, plain)

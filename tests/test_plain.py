@@ -205,6 +205,69 @@ def test_norm_placement_and_head():
     assert np.array_equal(plain.forward(wa2, cfg_a, [1, 2, 3]), xa)
 
 
+def _one_head_attention(cfg, q1, keys, values):
+    """``plain.attention_half`` of two tokens at position 0 (no rotation) with projections
+    that copy slices of the input: head 0's query is ``q1`` for the second token, the one
+    key/value head's keys and values are ``keys`` and ``values``, and the output is head
+    0's context.  Unit norm weights.  Returns the second token's context."""
+    nh, nkv, hd, H = (cfg[k] for k in ("num_attention_heads", "num_key_value_heads", "head_dim", "hidden_size"))
+    assert nkv == 1 and H >= 3 * hd
+    eye = np.eye(hd)
+    p = "model.layers.0"
+    w = {f"{p}.self_attn.q_proj.weight": np.zeros((nh * hd, H)), f"{p}.self_attn.k_proj.weight": np.zeros((hd, H)),
+         f"{p}.self_attn.v_proj.weight": np.zeros((hd, H)), f"{p}.self_attn.o_proj.weight": np.zeros((H, nh * hd)),
+         f"{p}.self_attn.q_norm.weight": np.ones(hd), f"{p}.self_attn.k_norm.weight": np.ones(hd)}
+    w[f"{p}.self_attn.q_proj.weight"][:hd, :hd] = eye          # head 0 of q = h[:, 0:hd]
+    w[f"{p}.self_attn.k_proj.weight"][:, hd:2 * hd] = eye       # k = h[:, hd:2hd]
+    w[f"{p}.self_attn.v_proj.weight"][:, 2 * hd:3 * hd] = eye   # v = h[:, 2hd:3hd]
+    w[f"{p}.self_attn.o_proj.weight"][:hd, :hd] = eye           # out[:, 0:hd] = context of head 0
+    h = np.zeros((2, H))
+    h[1, :hd] = q1
+    h[:, hd:2 * hd] = keys
+    h[:, 2 * hd:3 * hd] = values
+    out, _ = plain.attention_half(h, w, p, cfg, positions=[0, 0])
+    return out[1, :hd]
+
+
+def test_attention_scale_is_one_over_root_head_dim():
+    """B's head size (32) is not hidden / heads (16): a scale taken from the wrong one of the
+    two moves the softmax weight of the closed form below from 0.804 to 0.881."""
+    cfg = CONFIGS["B"]
+    hd, eps = cfg["head_dim"], cfg["rms_norm_eps"]
+    assert hd != cfg["hidden_size"] // cfg["num_attention_heads"]
+    a = np.ones(hd)
+    b = np.ones(hd)
+    b[:4] = -1.0  # a . b = hd - 8, both of unit mean square
+    values = rng.normal(size=(2, hd))
+    got = _one_head_attention(cfg, a, np.stack([b, a]), values)
+    # normed vectors are a, b / sqrt(1 + eps); scores differ by (a.a - a.b) / (1 + eps) * scale
+    delta = 8.0 / (1.0 + eps) / math.sqrt(hd)
+    weight = 1.0 / (1.0 + math.exp(-delta))
+    assert np.allclose(got, weight * values[1] + (1 - weight) * values[0], atol=1e-12)
+    wrong = 1.0 / (1.0 + math.exp(-8.0 / (1.0 + eps) / math.sqrt(cfg["hidden_size"] // cfg["num_attention_heads"])))
+    assert abs(weight - wrong) > 0.05
+
+
+def test_head_norms_use_the_configurations_eps():
+    """A query so small that eps decides its normed length: with B's 1e-5 the softmax weight
+    below is 0.605, with a fixed 1e-6 it would be 0.731."""
+    cfg = CONFIGS["B"]
+    hd, eps = cfg["head_dim"], cfg["rms_norm_eps"]
+    assert eps == 1e-5
+    t = 1e-3
+    a = np.ones(hd)
+    b = np.ones(hd)
+    b[:4] = -1.0
+    values = rng.normal(size=(2, hd))
+    got = _one_head_attention(cfg, t * a, np.stack([b, a]), values)
+    shrink = t / math.sqrt(t * t + eps)  # the normed query is shrink * a
+    delta = shrink * 8.0 / math.sqrt(1.0 + eps) / math.sqrt(hd)
+    weight = 1.0 / (1.0 + math.exp(-delta))
+    assert np.allclose(got, weight * values[1] + (1 - weight) * values[0], atol=1e-12)
+    other = 1.0 / (1.0 + math.exp(-(t / math.sqrt(t * t + 1e-6)) * 8.0 / math.sqrt(1.0 + eps) / math.sqrt(hd)))
+    assert abs(weight - other) > 0.05
+
+
 def test_schedule_names_a_layer_twice_and_borrows_a_cache():
     cfg = CONFIGS["A"]
     w = _weights(cfg, 7)

@@ -145,6 +145,44 @@ def test_a_stateful_toy_mixer_registers_builds_and_steps(tmp_path):
             g = np.concatenate(got[rid])
             assert np.abs(g - want[rid][: len(g)]).max() <= 2e-5 * np.abs(want[rid]).max(), rid
         assert pos == {"t0": 40, "t1": 23, "t2": 57}
+        for seq in list(live.values()):
+            runner.close(seq)
+
+        # a step that fails in the second layer, after the toy mixer has overwritten its state:
+        # pages, lengths and the state are as before it, and the request goes on correctly
+        toks = reqs["t0"]
+        seq = runner.open("again")
+        head = runner.step([StepEntry(seq, toks[:10], list(range(10)))]).cpu().numpy()
+        state_before = runner.manager.slots.tensors[0][seq.slot].clone()
+        free_before = runner.manager.free_pages
+        second = runner.model.blocks[1]
+        intact = second.forward
+
+        def broken(*args, **kwargs):
+            raise RuntimeError("the second layer failed")
+
+        second.forward = broken
+        try:
+            with pytest.raises(RuntimeError, match="second layer failed"):
+                runner.step([StepEntry(seq, toks[10:30], [])])
+        finally:
+            second.forward = intact
+        assert seq.length == 10 and runner.manager.free_pages == free_before
+        assert torch.equal(runner.manager.slots.tensors[0][seq.slot], state_before)
+        runner.manager.check()
+        rest = runner.step([StepEntry(seq, toks[10:], list(range(len(toks) - 10)))]).cpu().numpy()
+        runner.close(seq)
+        got_again = np.concatenate([head, rest])
+        assert np.abs(got_again - want["t0"]).max() <= 2e-5 * np.abs(want["t0"]).max()
+
+        # start-up takes the state's bytes off the budget before it counts pages
+        from pylon_amd.config import PylonConfig
+
+        sized = Runner.from_config(PylonConfig(model_path=str(folder), dtype="float32", page_size=16,
+                                               max_batch_size=3))
+        assert sized.pool_sizing["state_bytes"] == 3 * cfg["hidden_size"] * 4
+        assert sized.pool_sizing["bytes_per_token"] == 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * 4
+        assert sized.manager.num_pages == 3 * (cfg["max_position_embeddings"] // 16)
     finally:
         unregister_part("mixer", "leaky_sum")
         unregister_architecture("ToyLeakyForCausalLM")

@@ -73,6 +73,33 @@ def test_element_types_follow_what_is_stored(tmp_path):
     assert model.blocks[0].feed_forward.params["down"].dtype == torch.bfloat16
     # a float32 model takes everything as float32
     assert _load(folder, torch.float32).params["embed"].dtype == torch.float32
+    # start-up counts the weights with the types they will have, from the headers alone
+    from pylon_amd.engine.runner import weight_bytes
+    from pylon_amd.weights.loader import stored_param_dtypes
+
+    arch, cfg = load_model_config(folder)
+    spec = arch.model_spec(cfg)
+    meta = Model(spec, dtype=torch.bfloat16, device="meta")
+    dtypes = stored_param_dtypes(meta, arch, cfg, folder)
+    assert dtypes["layers.1.feed_forward.down"] == torch.float32
+    assert dtypes["layers.0.feed_forward.down"] == torch.bfloat16 and dtypes["final_norm.weight"] == torch.float32
+    extra = 2 * down.numel()  # two more bytes for each of its elements
+    assert weight_bytes(spec, torch.bfloat16, dtypes) == weight_bytes(spec, torch.bfloat16) + extra
+    real = sum(o.params[n].numel() * o.params[n].element_size() for _, o, n in model.named_params())
+    assert weight_bytes(spec, torch.bfloat16, dtypes) == real
+
+
+def test_matrices_kept_in_32_bit_are_reported(tmp_path, caplog):
+    folder = make_model_folder(tmp_path, "A", dtype="float32")
+    with caplog.at_level("WARNING", logger="pylon"):
+        model = _load(folder, torch.bfloat16)
+    assert model.params["embed"].dtype == torch.float32
+    assert "weights_kept_32bit" in caplog.text and "twice the memory" in caplog.text
+    caplog.clear()
+    with caplog.at_level("WARNING", logger="pylon"):
+        _load(folder, torch.float32)
+        _load(make_model_folder(tmp_path, "A", dtype="bfloat16"), torch.bfloat16)
+    assert "weights_kept_32bit" not in caplog.text
 
 
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
