@@ -9,7 +9,8 @@ Interfaces
 norm          ``forward(x) -> y`` and ``add_forward(resid, delta, row_idx=None) -> y``:
               ``resid`` is the float32 residual stream, ``delta`` the previous part's
               output (or None), either ``[tokens, dim]`` or a stack ``[parts, tokens, dim]``
-              of float32 partial sums still to be added up; the sum is formed in float32, stored back into
+              of float32 partial sums still to be added up (:func:`summed` makes one float32
+              tensor of either); the sum is formed in float32, stored back into
               ``resid`` (unless ``row_idx`` picks rows), and its norm is returned in
               the activation dtype.
 position      ``rotary() -> (inv_freq, rotary_dim) | None`` for encodings applied by
@@ -54,6 +55,18 @@ class StateRequirement:
 
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+
+
+def summed(delta: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """A part's output that has not been added to the residual stream yet, as one float32
+    ``[tokens, dim]`` tensor.  What a mixer or a feed-forward hands on is either a tensor of
+    that shape in the activation dtype or a stack ``[parts, tokens, dim]`` of float32 partial
+    sums (the product kernels cut the reduction over workgroups for some row counts); which
+    of the two depends on the step's size, so a norm or a block that adds it up itself goes
+    through this function (the built-in norm kernel takes both forms directly)."""
+    if delta is None:
+        return None
+    return delta.sum(dim=0) if delta.dim() == 3 else delta.float()
 
 
 class Part:

@@ -28,15 +28,8 @@ class CentredNormSpec:
 def build_toys():
     from pylon_amd.config.registry import Architecture, WeightTarget
     from pylon_amd.models import qwen3
-    from pylon_amd.parts.base import Part
+    from pylon_amd.parts.base import Part, summed
     from pylon_amd.parts.registry import build_part
-
-    def summed(delta):
-        """A part's output that has not been added yet: a tensor of the residual's shape, or
-        a stack of float partial sums."""
-        if delta is None:
-            return None
-        return delta.sum(dim=0) if delta.dim() == 3 else delta.float()
 
     class CentredNorm(Part):
         """y = (x - mean) / sqrt(var + eps) * weight + bias, in float32, rounded once."""
