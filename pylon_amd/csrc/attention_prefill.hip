@@ -380,12 +380,10 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
     int page_size, int window, float scale) {
   constexpr int HD = 128, KS = HD / 32, DT = HD / 16;
   constexpr int ROW = HD * 2;  // bytes of a key or value row in LDS
-  constexpr int TILE = AP_BK * HD;  // elements of a block of keys or values
-  __shared__ __attribute__((aligned(16))) uint16_t kv_lds[4 * TILE];
-  uint16_t* const k_a = kv_lds;
-  uint16_t* const k_b = k_a + TILE;
-  uint16_t* const v_a = k_a + 2 * TILE;
-  uint16_t* const v_b = k_a + 3 * TILE;
+  __shared__ __attribute__((aligned(16))) uint16_t k_a[AP_BK * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t k_b[AP_BK * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t v_a[AP_BK * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t v_b[AP_BK * HD];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -445,7 +443,6 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
     }                                                                                                  \
   } while (0)
 
-  const int kb_end = ((kv_last - kb_first) / AP_BK) * AP_BK + kb_first;  // the last block
   APD_FETCH(kb_first, k_a, v_a);
 
   int qpos[QT];
@@ -471,10 +468,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
   do {                                                                                                 \
     __builtin_amdgcn_s_waitcnt(0);                                                                     \
     __syncthreads();                                                                                   \
-    /* never taken (the loop ends at kb_end); with the math under a condition the compiler holds */    \
-    /* some forty registers fewer (206 against 244 at 128 rows), and the kernel runs 8 % faster */     \
-    if ((KB) > kb_end) break;                                                                          \
-    if ((KB) + AP_BK <= kb_end) APD_FETCH((KB) + AP_BK, KNEXT, VNEXT);                                 \
+    if ((KB) + AP_BK <= kv_last) APD_FETCH((KB) + AP_BK, KNEXT, VNEXT);                                \
     const AP_LDS(char)* k_tile = (const AP_LDS(char)*)(KCUR);                                          \
     const AP_LDS(char)* v_tile = (const AP_LDS(char)*)(VCUR);                                          \
     /* scores: the operands of the next 16 keys are read while this tile's products run */             \
@@ -552,9 +546,9 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
 
   for (int kb = kb_first;; kb += 2 * AP_BK) {
     APD_BLOCK(kb, k_a, v_a, k_b, v_b);
-    if (kb + AP_BK > kb_end) break;
+    if (kb + AP_BK > kv_last) break;
     APD_BLOCK(kb + AP_BK, k_b, v_b, k_a, v_a);
-    if (kb + 2 * AP_BK > kb_end) break;
+    if (kb + 2 * AP_BK > kv_last) break;
   }
 #undef APD_BLOCK
 #undef APD_FETCH

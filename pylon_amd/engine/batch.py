@@ -118,7 +118,7 @@ class StepContext:
     chosen: Optional[torch.Tensor] = None  # int32 [slots]: last sampled token per state slot
     logits_out: Optional[torch.Tensor] = None  # float32 [>= n_logits, vocab]: where the logits go, if given
     arena: Optional[MetadataArena] = None  # pinned staging for what parts put on the device themselves
-    _tiles: Dict[Tuple[int, int], torch.Tensor] = field(default_factory=dict)
+    _tiles: Dict[Tuple[int, int, int], torch.Tensor] = field(default_factory=dict)
 
     def cache(self, cache_id: int) -> CacheView:
         return self.views[cache_id]
@@ -130,12 +130,15 @@ class StepContext:
         more = np.nonzero(self.counts != 1)[0]
         return int(more[0]) if more.size else self.rows
 
-    def token_tiles(self, tokens_per_tile: int, skip_rows: int = 0) -> torch.Tensor:
+    def token_tiles(self, tokens_per_tile: int, skip_rows: int = 0, fold: int = 0) -> torch.Tensor:
         """int32 ``[n, 4]`` on the device: the step's tokens (without those of the first
         ``skip_rows`` rows) cut into runs of at most ``tokens_per_tile`` consecutive tokens
         of one row, as (index of the first token, count, row, position of the first token),
-        longest context first so that the heaviest tiles start first."""
-        key = (tokens_per_tile, skip_rows)
+        longest context first so that the heaviest tiles start first.  With ``fold`` (the
+        number of tiles whose workgroups fill the chip once) every second run of ``fold``
+        tiles is turned round: where two workgroups share a compute unit, the one that
+        arrives second beside the heaviest of a round is the lightest of the next."""
+        key = (tokens_per_tile, skip_rows, fold)
         tiles = self._tiles.get(key)
         if tiles is None:
             per_row = -(-self.counts // tokens_per_tile)
@@ -149,6 +152,9 @@ class StepContext:
             np.cumsum(self.counts, out=starts[1:])
             table = np.stack([starts[row] + within, count, row, self.starts[row] + within], axis=1)
             order = np.argsort(-(table[:, 3] + table[:, 1]), kind="stable")
+            if fold > 0:
+                for start in range(fold, len(order), 2 * fold):
+                    order[start: start + fold] = order[start: start + fold][::-1].copy()
             ordered = table[order].astype(np.int32)
             if self.arena is not None:
                 tiles = self.arena.stage(ordered)

@@ -17,20 +17,6 @@ from .base import KVRequirement, Part
 from .registry import build_part, register_part
 
 
-# In a step that carries decoding requests beside prompt portions, the decode kernel runs on a
-# second stream beside the prompt kernel (measured at the Qwen3-4B sizes, 64 requests of 4,096
-# cached tokens beside a 2,048-token portion: 28.4 -> 27.5 ms a step).
-OVERLAP_MIXED_ATTENTION = True
-_side_streams = {}
-
-
-def _side_stream(device) -> "torch.cuda.Stream":
-    stream = _side_streams.get(device)
-    if stream is None:
-        stream = _side_streams[device] = torch.cuda.Stream(device=device)
-    return stream
-
-
 class Attention(Part):
     def __init__(self, spec: AttentionSpec, *, dtype: torch.dtype, device) -> None:
         super().__init__()
@@ -113,7 +99,7 @@ class Attention(Part):
             singles = ctx.leading_singles
             if not (0 < singles <= ops.DECODE_MAX_TOKENS and ops.decode_attention_ok(q[:singles], cache.k)):
                 singles = 0
-            def decode_part():
+            if singles:
                 span = int(ctx.starts[:singles].max()) + 1
                 if spec.window is not None:
                     span = min(span, spec.window)
@@ -123,29 +109,12 @@ class Attention(Part):
                     page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits,
                     n_cuts=cuts, out=context[:singles],
                 )
-
-            def prompt_part():
-                tiles = ctx.token_tiles(rows // group, skip_rows=singles)
+            if singles < ctx.rows:
+                tiles = ctx.token_tiles(rows // group, skip_rows=singles, fold=ops.prefill_fold(spec.n_kv_heads))
                 ops.attention_prefill(
                     q, cache.k, cache.v, cache.block_table, tiles,
                     page_size=cache.page_size, window=spec.window, scale=spec.scale, rows=rows, out=context,
                 )
-
-            if singles and singles < ctx.rows and OVERLAP_MIXED_ATTENTION:
-                # The decoding requests read their keys (bound by memory) while the prompt
-                # portions multiply theirs (bound by the matrix cores): side by side.
-                main = torch.cuda.current_stream()
-                side = _side_stream(h.device)
-                side.wait_stream(main)
-                with torch.cuda.stream(side):
-                    decode_part()
-                prompt_part()
-                main.wait_stream(side)
-            else:
-                if singles:
-                    decode_part()
-                if singles < ctx.rows:
-                    prompt_part()
         else:
             context = ops.paged_attention(
                 q, cache.k, cache.v, cache.block_table, ctx.tok_row, ctx.positions,

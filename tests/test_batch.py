@@ -41,3 +41,19 @@ def test_tiles_cover_every_token_once_longest_context_first():
             _check_cover(tiles, counts, cached, per_tile, skip)
             ends = (tiles[:, 3] + tiles[:, 1]).tolist()
             assert ends == sorted(ends, reverse=True)
+
+
+def test_folded_tiles_turn_every_second_run_round():
+    counts, cached = [1, 1, 37, 5, 64, 130], [9, 0, 0, 31, 16, 3]
+    ctx = _step(counts, cached)
+    plain = (lambda t: (t[:, 3] + t[:, 1]).tolist())(ctx.token_tiles(4, skip_rows=2))
+    for fold in (1, 3, 5, 1000):
+        tiles = ctx.token_tiles(4, skip_rows=2, fold=fold)
+        _check_cover(tiles, counts, cached, 4, 2)
+        ends = (tiles[:, 3] + tiles[:, 1]).tolist()
+        want = []
+        for start in range(0, len(plain), fold):
+            run = plain[start: start + fold]
+            want += run[::-1] if (start // fold) % 2 else run
+        assert ends == want
+    assert ctx.token_tiles(4, skip_rows=2, fold=1000).tolist() == ctx.token_tiles(4, skip_rows=2).tolist()
