@@ -189,9 +189,10 @@ __global__ __launch_bounds__(512) void rmsnorm_kernel(TO* __restrict__ out, TX* 
 // row's stores travel beside the next row's loads instead of every workgroup of the launch
 // reading at one time and writing at another (2,048 rows of 2,560: 19.5 -> 15.8 us on data
 // that no cache holds; four rows per workgroup lose again, 19.2 us).  Float residual, one
-// delta, rows of a multiple of 4 elements that fit 16 per thread.
-template <typename TD, typename TO, int R>
-__global__ __launch_bounds__(256) void add_rmsnorm_many_kernel(TO* __restrict__ out, float* resid,
+// delta, rows of a multiple of 4 elements that fit 16 per thread; as many threads as the
+// kernel for few rows has at this width, so that a row's sum is formed in the same order.
+template <typename TD, typename TO, int R, int THREADS>
+__global__ __launch_bounds__(THREADS) void add_rmsnorm_many_kernel(TO* __restrict__ out, float* resid,
                                                                const TD* __restrict__ delta,
                                                                const float* __restrict__ w, int rows, int dim,
                                                                float eps) {
@@ -203,7 +204,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_many_kernel(TO* __restrict__ 
   const int r0 = blockIdx.x * R;
 #pragma unroll
   for (int n = 0; n < VEC; ++n) {
-    const int c = threadIdx.x + n * 256;
+    const int c = threadIdx.x + n * THREADS;
     wt[n] = (c < chunks) ? w4[c] : float4{0.f, 0.f, 0.f, 0.f};
   }
 #pragma unroll
@@ -213,7 +214,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_many_kernel(TO* __restrict__ 
     const TD* dr = delta + static_cast<size_t>(live ? r0 + i : r0) * dim;
 #pragma unroll
     for (int n = 0; n < VEC; ++n) {
-      const int c = threadIdx.x + n * 256;
+      const int c = threadIdx.x + n * THREADS;
       if (c < chunks) {
         const float4 x = reinterpret_cast<const float4*>(xr)[c];
         const float4 d = load4(dr, c);
@@ -237,7 +238,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_many_kernel(TO* __restrict__ 
     TO* yr = out + static_cast<size_t>(r0 + i) * dim;
 #pragma unroll
     for (int n = 0; n < VEC; ++n) {
-      const int c = threadIdx.x + n * 256;
+      const int c = threadIdx.x + n * THREADS;
       if (c < chunks) {
         reinterpret_cast<float4*>(xr)[c] = held[i][n];
         store4(yr, c, (held[i][n].x * inv) * wt[n].x, (held[i][n].y * inv) * wt[n].y,
@@ -255,15 +256,18 @@ static void launch_rmsnorm_out(void* out, int out_dtype, TX* x, const TD* delta,
                                int dim, float eps, int write_resid, hipStream_t stream) {
   if constexpr (sizeof(TX) == 4) {
     if (rows >= PYLON_NORM_MANY_ROWS && delta != nullptr && n_delta == 1 && row_idx == nullptr && write_resid &&
-        (dim & 3) == 0 && dim <= 4096) {
+        (dim & 3) == 0 && dim <= 8192) {
       constexpr int R = 2;
-      dim3 grid((rows + R - 1) / R), block(256);
-      if (out_dtype == PYLON_F32)
-        hipLaunchKernelGGL((add_rmsnorm_many_kernel<TD, float, R>), grid, block, 0, stream, (float*)out, x, delta, w,
-                           rows, dim, eps);
-      else
-        hipLaunchKernelGGL((add_rmsnorm_many_kernel<TD, bf16_t, R>), grid, block, 0, stream, (bf16_t*)out, x, delta,
-                           w, rows, dim, eps);
+      dim3 grid((rows + R - 1) / R);
+#define GO(TO, THREADS)                                                                                    \
+  hipLaunchKernelGGL((add_rmsnorm_many_kernel<TD, TO, R, THREADS>), grid, dim3(THREADS), 0, stream, (TO*)out, x, \
+                     delta, w, rows, dim, eps)
+      if (dim > 4096) {
+        if (out_dtype == PYLON_F32) GO(float, 512); else GO(bf16_t, 512);
+      } else {
+        if (out_dtype == PYLON_F32) GO(float, 256); else GO(bf16_t, 256);
+      }
+#undef GO
       return;
     }
   }

@@ -109,6 +109,28 @@ def test_rmsnorm_and_fused_residual(ops, dtype, dim):
     assert np.abs(f64(r2) - summed).max() <= 1e-6 * np.abs(summed).max()
 
 
+@pytest.mark.parametrize("dim", [80, 2560 + 16, 5120 + 8, 8192])
+@pytest.mark.parametrize("delta_dtype", DTYPES)
+def test_residual_norm_of_many_rows_has_the_bits_of_few(ops, dim, delta_dtype):
+    """From 512 rows on another kernel takes the fused residual norm (two rows a workgroup):
+    it forms every row's sums in the order of the kernel for few rows, so a request's values do
+    not depend on how many tokens share its step."""
+    eps, rows = 1e-6, 515
+    x = rnd((rows, dim), 60, torch.float32, 2.0)
+    delta = rnd((rows, dim), 61, delta_dtype)
+    w = 1 + 0.3 * rnd((dim,), 62)
+    summed = f64(x) + f64(delta)
+    want = summed / np.sqrt((summed * summed).mean(-1, keepdims=True) + eps) * f64(w)
+    for out_dtype in DTYPES:
+        many_resid = x.clone().to(DEV)
+        many = ops.add_rmsnorm(many_resid, delta.to(DEV), w.to(DEV), eps, out_dtype)
+        assert np.abs(f64(many) - want).max() <= tol(out_dtype, np.abs(want).max())
+        for lo, hi in ((0, 3), (200, 201), (513, 515)):
+            few_resid = x[lo:hi].clone().to(DEV)
+            few = ops.add_rmsnorm(few_resid, delta[lo:hi].contiguous().to(DEV), w.to(DEV), eps, out_dtype)
+            assert torch.equal(few, many[lo:hi]) and torch.equal(few_resid, many_resid[lo:hi])
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_silu_gate(ops, dtype):
     gu = rnd((5, 2 * 176), 5, dtype, 3.0)
