@@ -195,6 +195,8 @@ class Engine:
         from .runner import Runner
 
         threaded = options.pop("threaded", False)
+        if config is not None and options:
+            raise TypeError("give the serving options as `config` or as keywords, not both")
         config = config if config is not None else PylonConfig(**options)
         runner = Runner.from_random(model_config, seed, config, std=std, norm_jitter=norm_jitter, draw_on=draw_on)
         return cls(config, runner=runner, threaded=threaded)
