@@ -199,3 +199,55 @@ def test_random_weights_start_up_like_a_folder(gpu):
     assert outputs[0] == outputs[1] and len(outputs[0]) == 6
     with pytest.raises(RuntimeError, match="Refusing to load a model of random weights"):
         Engine.from_random(CONFIGS["D"], 5, max_gpu_utilization=1e-9)
+
+
+def test_groups_of_runs_get_pages_of_their_own_at_start_up(gpu, tmp_path):
+    """A toy architecture (Qwen3's parts, the first layer with a window of 40 tokens): the sized
+    pool gives the windowed group only the pages it can ever use, the engine runs long
+    requests side by side through it without running out, and the tokens are the plain model's."""
+    import dataclasses
+
+    from pylon_amd.config import register_architecture, unregister_architecture
+    from pylon_amd.config.registry import Architecture
+    from pylon_amd.engine.engine import Engine
+    from pylon_amd.models import qwen3
+    from pylon_amd.sampling import Sampling
+    from pylon_amd.weights import write_random_model
+
+    def model_spec(cfg):
+        spec = qwen3.model_spec(cfg)
+        layers = list(spec.layers)
+        layers[0] = dataclasses.replace(layers[0], mixer=dataclasses.replace(layers[0].mixer, window=40))
+        return dataclasses.replace(spec, layers=tuple(layers))
+
+    arch = Architecture("ToyWindowedForCausalLM", qwen3.parse_config, model_spec, qwen3.weight_targets,
+                        lambda cfg: dict(qwen3.config_to_json(cfg), architectures=["ToyWindowedForCausalLM"]))
+    register_architecture(arch)
+    try:
+        config = dict(CONFIGS["C"], architectures=["ToyWindowedForCausalLM"])
+        folder = write_random_model(tmp_path / "windowed", config, 9, dtype="float32", std=0.08, norm_jitter=0.2)
+        cfg, weights = read_folder(folder)
+        engine = Engine.from_folder(folder, dtype="float32", page_size=16, max_batch_size=3, prefill_chunk_size=32)
+        try:
+            manager = engine.runner.manager
+            # the full group: three requests of 2,048 positions; the windowed one: per request the
+            # pages of 40 + 32 tokens and one more
+            assert engine.runner.pool_sizing["pages_per_group"] == [18, 3 * 128]
+            assert [g.requirement.window for g in manager.groups] == [40, None]
+            assert [g.pool.num_pages for g in manager.groups] == [18, 384] and manager.num_pages == 384
+            prompts = [random_tokens(cfg["vocab_size"], n, 20 + n) for n in (210, 77, 300, 150)]
+            results = engine.generate(prompts, Sampling(max_new_tokens=30, temperature=0.0))
+            assert manager.groups[0].pool.free_pages == 18 and manager.groups[1].pool.free_pages == 384
+            manager.check()
+        finally:
+            engine.close()
+        for prompt, result in zip(prompts, results):
+            assert len(result.output_ids) == 30
+            ref = list(prompt)
+            for got in result.output_ids:
+                row = plain.forward(weights, cfg, ref, windows={0: 40})[-1]
+                best = np.sort(row)
+                assert got == int(row.argmax()) or best[-1] - row[got] <= 1e-4 * np.abs(row).max()
+                ref.append(got)
+    finally:
+        unregister_architecture("ToyWindowedForCausalLM")
