@@ -64,14 +64,14 @@ def causal_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float,
     group = heads // k.shape[0]
     k = np.repeat(k, group, axis=0)
     v = np.repeat(v, group, axis=0)
-    scores = np.einsum("hid,hjd->hij", q, k) * scale
+    scores = (q @ k.transpose(0, 2, 1)) * scale  # [heads, T, T]
     i = np.arange(tokens)[:, None]
     j = np.arange(tokens)[None, :]
     visible = j <= i
     if window is not None:
         visible &= j > i - window
     scores = np.where(visible[None], scores, -np.inf)
-    return np.einsum("hij,hjd->hid", softmax(scores, axis=-1), v)
+    return softmax(scores, axis=-1) @ v
 
 
 def silu(x: np.ndarray) -> np.ndarray:
