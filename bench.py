@@ -293,6 +293,8 @@ def main() -> int:
     parser.add_argument("--shape", choices=sorted(SHAPES), default="4b", help="layer sizes (default: Qwen3-4B)")
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has")
     parser.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens cached before decoding starts")
+    parser.add_argument("--context-length", type=int, default=None,
+                        help="longest request in tokens (default: the shape's max_position_embeddings)")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
     parser.add_argument("--no-points", action="store_true", help="skip the other batch sizes and contexts")
@@ -313,7 +315,9 @@ def main() -> int:
         return 1
     from pylon_amd.engine import Runner
 
-    shape = SHAPES[args.shape]
+    shape = dict(SHAPES[args.shape])
+    if args.context_length:
+        shape["max_position_embeddings"] = args.context_length
     layers = args.layers or shape["num_hidden_layers"]
     context_length = shape["max_position_embeddings"]
     prompt_len = args.prompt_len
