@@ -20,6 +20,15 @@
 // per chunk, preceded by a counted wait for this wave's loads of chunk c only, so the later
 // loads stay in flight across it.  No sums cross waves: a wave owns its columns.
 //
+// A workgroup takes `wg_cols` columns, at most what its waves' tiles hold and not necessarily
+// that many: the host gives every workgroup of a launch the same share of the columns, chosen
+// so that the workgroups are a whole number of rounds over the compute units.  Its waves take
+// full tiles in turn; the rows of a tile beyond the workgroup's columns are out of range and
+// fetch nothing, and a wave left without columns only helps to bring the rows of x.  (The
+// gate/up product of 2 x 9728 columns: 38 per workgroup, one workgroup per unit, 20.0 us
+// against 21.0 for 64 or 48 columns per workgroup where some units stream half as much again
+// as others.)
+//
 // All loads go through buffer descriptors (of the workgroup's rows of w; of x): rows beyond
 // N or M and elements beyond K are read as zeros without a memory access and without a
 // branch, so every wave issues the same number of loads per chunk and the counted waits
@@ -68,7 +77,7 @@ template <int MT, int CT, bool GLU, int WAVES, typename TO>
 __device__ __forceinline__ void gemm_rows_body(
     TO* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int M, int N,
     int K, long long ldx, long long ldw, long long ldo, long long part_stride, int chunks_per_part,
-    int spread) {
+    int wg_cols) {
   typedef GrShape<MT, CT, WAVES> Shape;
   constexpr int QW = 4 / WAVES;  // quarters of every tile of x that a wave fills
   constexpr int STAGES = Shape::STAGES;
@@ -79,21 +88,18 @@ __device__ __forceinline__ void gemm_rows_body(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PYLON_WAVE);
   const int r = lane & 15, g = lane >> 4;
   constexpr int WAVE_COLS = (GLU ? 1 : CT) * 16;  // columns of the output per wave
-  constexpr int WG_COLS = WAVES * WAVE_COLS;
-  // A workgroup's waves take neighbouring groups of columns, or, spread, groups that lie
-  // gridDim.x apart: a matrix of 608 groups then keeps 256 workgroups (two or three waves
-  // of each) busy instead of 152.
-  const int wg_row0 = spread ? 0 : blockIdx.x * WG_COLS;  // first row of w the descriptor covers
-  const int n0 = spread ? (blockIdx.x + gridDim.x * wave) * WAVE_COLS : wg_row0 + wave * WAVE_COLS;
+  const int wg_row0 = blockIdx.x * wg_cols;  // first row of w the descriptor covers
+  const int wg_end = (N - wg_row0 < wg_cols) ? N : wg_row0 + wg_cols;
+  const int n0 = wg_row0 + wave * WAVE_COLS;
+  const int n_end = (wg_end - n0 < WAVE_COLS) ? wg_end : n0 + WAVE_COLS;  // <= n0: a wave without columns
   const int part = blockIdx.y;
   const int chunks = (K + GR_CHUNK - 1) / GR_CHUNK;
   const int c_begin = part * chunks_per_part;
   const int c_end = (c_begin + chunks_per_part < chunks) ? c_begin + chunks_per_part : chunks;
 
   // The descriptor of w starts at the workgroup's first row (with GLU it reaches N rows
-  // further, to its up rows; spread, it covers the matrix: the host checks that this fits
-  // 31 bits).
-  const int wg_rows = (spread || N - wg_row0 < WG_COLS) ? N - wg_row0 : WG_COLS;
+  // further, to its up rows).
+  const int wg_rows = wg_end - wg_row0;
   const __amdgpu_buffer_rsrc_t wres = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t*>(w + static_cast<size_t>(wg_row0) * ldw), 0,
       static_cast<int>((static_cast<long long>((GLU ? N : 0) + wg_rows - 1) * ldw + K) * 2), 0x00020000);
@@ -128,7 +134,7 @@ __device__ __forceinline__ void gemm_rows_body(
       // the row within the workgroup's columns, and where it lies from the descriptor's base
       const int col = n0 - wg_row0 + (GLU ? R : 16 * j + R);
       const unsigned row = static_cast<unsigned>(col) + ((GLU && j == 1) ? static_cast<unsigned>(N) : 0u);
-      w_at[j][q] = (wg_row0 + col < N) ? row * static_cast<unsigned>(ldw) * 2u + 2u * w_k[q] : GR_OOB;
+      w_at[j][q] = (wg_row0 + col < n_end) ? row * static_cast<unsigned>(ldw) * 2u + 2u * w_k[q] : GR_OOB;
     }
   }
   // Operand reads: lane (r, g) takes piece 4 s + g of row r of a tile.
@@ -197,7 +203,7 @@ __device__ __forceinline__ void gemm_rows_body(
     gr_wait_loads<LOADS*(STAGES - 2)>();
     gr_barrier();
     issue(c + STAGES - 1, stage == 0 ? STAGES - 1 : stage - 1);
-    compute(stage);
+    if (n0 < n_end) compute(stage);
     stage = (stage + 1 == STAGES) ? 0 : stage + 1;
   }
   // The loads still outstanding are those past the range: they fetch nothing but do write
@@ -223,7 +229,7 @@ __device__ __forceinline__ void gemm_rows_body(
         for (int i = 0; i < 4; ++i) v[i] = gr_silu(acc[0][t][i]) * acc[1][t][i];
       }
       TO* p = dst + static_cast<size_t>(m) * ldo + n;
-      if (wide && n + 3 < N) {
+      if (wide && n + 3 < n_end && (n & 3) == 0) {
         if constexpr (sizeof(TO) == 4) {
           *reinterpret_cast<floatx4*>(p) = v;
         } else {
@@ -235,7 +241,7 @@ __device__ __forceinline__ void gemm_rows_body(
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (n + i < N) p[i] = from_float<TO>(v[i]);
+          if (n + i < n_end) p[i] = from_float<TO>(v[i]);
       }
     }
   }
@@ -245,30 +251,40 @@ template <int MT, int CT, bool GLU, int WAVES, typename TO>
 __global__ __launch_bounds__(WAVES* PYLON_WAVE) void gemm_rows_kernel(
     TO* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int M, int N,
     int K, long long ldx, long long ldw, long long ldo, long long part_stride, int chunks_per_part,
-    int spread) {
-  gemm_rows_body<MT, CT, GLU, WAVES, TO>(out, x, w, M, N, K, ldx, ldw, ldo, part_stride, chunks_per_part, spread);
+    int wg_cols) {
+  gemm_rows_body<MT, CT, GLU, WAVES, TO>(out, x, w, M, N, K, ldx, ldw, ldo, part_stride, chunks_per_part, wg_cols);
 }
 
 // How a product is laid over the chip: wavefronts per workgroup, workgroups along the columns,
-// and whether a workgroup's waves take column groups that lie `groups` apart.
+// and the columns each of them takes.
 struct GrLaunch {
-  int waves, groups, spread;
+  int waves, groups, wg_cols;
 };
 
 // units: compute units of the device.  waves: 4, 2, or 0 for two where four would give fewer
-// workgroups than half the units.
-static GrLaunch gr_launch_shape(int N, long long ldw, int parts, int col_tiles, int glu, int waves, int units) {
+// workgroups than half the units.  cols: columns per workgroup, or 0 for the rule: an equal
+// share for every workgroup of as many whole rounds over the units as workgroups of full
+// width would need (at least 16 columns), unless that makes the workgroups re-read more rows
+// of x than they stream rows of w; then, and beyond 16 rows of x in launches of several rounds,
+// the full width.  Measured at 2560 x 9728, K cut in eight, 32 rows: 13.2 us with 80 columns
+// (256 workgroups) against 14.9 with 128 (160); 2560 x 4096 cut in four, 48 rows: 9.15 with
+// 40 columns against 9.08 with 64; the head of 151936 rows at 8 rows of x: 136.5 with 119
+// columns against 141; at 64 rows of x: 181 against 170.5.
+static GrLaunch gr_launch_shape(int M, int N, int parts, int col_tiles, int glu, int waves, int units, int cols) {
   const int wave_cols = (glu ? 1 : col_tiles) * 16;
   if (waves == 0)
     waves = (static_cast<long long>((N + 4 * wave_cols - 1) / (4 * wave_cols)) * parts < units / 2) ? 2 : 4;
-  const int tasks = (N + wave_cols - 1) / wave_cols;  // groups of columns, one per wave
-  int groups = (tasks + waves - 1) / waves;
-  // Between `units` and `units * waves` groups of a matrix that one descriptor can cover: one
-  // workgroup per compute unit, whose waves take groups `units` apart.
-  const int spread = parts == 1 && tasks > units && groups < units &&
-                     static_cast<long long>(glu ? 2 * N : N) * ldw * 2 < (1ll << 31);
-  if (spread) groups = units;
-  return GrLaunch{waves, groups, spread};
+  const int full = waves * wave_cols;
+  if (cols <= 0) {
+    const long long least = static_cast<long long>((N + full - 1) / full) * parts;  // workgroups of full width
+    const long long rounds = (least + units - 1) / units;
+    const long long groups = rounds * units / parts;
+    int even = groups > 0 ? static_cast<int>((N + groups - 1) / groups) : full;
+    even = even < 16 ? 16 : (even > full ? full : even);
+    const bool pays = M <= 16 || (rounds == 1 && even * (glu ? 2 : 1) >= M);
+    cols = pays ? even : full;
+  }
+  return GrLaunch{waves, (N + cols - 1) / cols, cols};
 }
 
 template <int MT, int CT, bool GLU, int WAVES>
@@ -277,16 +293,15 @@ static void launch_rows_waves(void* out, int out_dtype, const void* x, const voi
                               const GrLaunch& shape, hipStream_t stream) {
   const int chunks = (K + GR_CHUNK - 1) / GR_CHUNK;
   const int per_part = (chunks + parts - 1) / parts;
-  const int groups = shape.groups, spread = shape.spread;
-  dim3 grid(groups, parts), block(WAVES * PYLON_WAVE);
+  dim3 grid(shape.groups, parts), block(WAVES * PYLON_WAVE);
   if (out_dtype == PYLON_F32)
     hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, GLU, WAVES, float>), grid, block, 0, stream, (float*)out,
                        (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part,
-                       spread);
+                       shape.wg_cols);
   else
     hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, GLU, WAVES, bf16_t>), grid, block, 0, stream, (bf16_t*)out,
                        (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part,
-                       spread);
+                       shape.wg_cols);
 }
 
 // Workgroups of four waves, or of two where four would leave compute units without one.
@@ -302,17 +317,17 @@ static void launch_rows(void* out, int out_dtype, const void* x, const void* w, 
 
 // What pylon_gemm_rows would launch for these arguments on a device of `units` compute units
 // (0: the current device's): shape[0] wavefronts per workgroup, shape[1] workgroups along
-// the columns (times `parts` along K), shape[2] whether the waves' column groups are spread.
+// the columns (times `parts` along K), shape[2] the columns each of them takes.
 // Touches no device memory; with units given it runs without a GPU.
-extern "C" int pylon_gemm_rows_shape(int N, long long ldw, int parts, int col_tiles, int glu, int waves,
-                                     int units, int* shape) {
-  PYLON_REQUIRE(shape != nullptr && N > 0 && parts >= 1, "gemm_rows_shape: bad arguments");
+extern "C" int pylon_gemm_rows_shape(int M, int N, int parts, int col_tiles, int glu, int waves, int units,
+                                     int cols, int* shape) {
+  PYLON_REQUIRE(shape != nullptr && M >= 1 && N > 0 && parts >= 1 && cols >= 0, "gemm_rows_shape: bad arguments");
   PYLON_REQUIRE(col_tiles == 1 || col_tiles == 2, "gemm_rows_shape: col_tiles is 1 or 2");
   PYLON_REQUIRE(waves == 0 || waves == 2 || waves == 4, "gemm_rows_shape: waves is 0, 2 or 4");
   if (units <= 0) units = pylon_compute_units();
   PYLON_REQUIRE(units > 0, "gemm_rows_shape: no device to take the number of compute units from");
-  const GrLaunch l = gr_launch_shape(N, ldw, parts, col_tiles, glu, waves, units);
-  shape[0] = l.waves, shape[1] = l.groups, shape[2] = l.spread;
+  const GrLaunch l = gr_launch_shape(M, N, parts, col_tiles, glu, waves, units, cols);
+  shape[0] = l.waves, shape[1] = l.groups, shape[2] = l.wg_cols;
   return 0;
 }
 
@@ -320,10 +335,12 @@ extern "C" int pylon_gemm_rows_shape(int N, long long ldw, int parts, int col_ti
 // up rows); out: `parts` results [M, ldo] spaced part_stride elements apart (parts > 1 needs
 // float out and no glu).  col_tiles: tiles of 16 columns per wave, 1 or 2; with glu a wave
 // takes 16 gate rows and their 16 up rows.  waves: wavefronts per workgroup, 4 or 2 (0: two if
-// four would give fewer workgroups than half the device's compute units).
+// four would give fewer workgroups than half the device's compute units).  cols: columns per
+// workgroup, at most what its waves' tiles hold (0: the rule of gr_launch_shape); the sums do
+// not depend on it.
 extern "C" int pylon_gemm_rows(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                                long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
-                               int col_tiles, int glu, int waves, hipStream_t stream) {
+                               int col_tiles, int glu, int waves, int cols, hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(out_dtype), "gemm_rows: unknown output dtype");
   PYLON_REQUIRE(M >= 0 && M <= 64, "gemm_rows: takes at most 64 rows, got %d", M);
   PYLON_REQUIRE(N > 0 && K > 0, "gemm_rows: bad sizes N=%d K=%d", N, K);
@@ -347,7 +364,9 @@ extern "C" int pylon_gemm_rows(void* out, int out_dtype, const void* x, const vo
   if (M == 0) return 0;
   const int units = pylon_compute_units();
   PYLON_REQUIRE(units > 0, "gemm_rows: the device's number of compute units is unknown");
-  const GrLaunch shape = gr_launch_shape(N, ldw, parts, col_tiles, glu, waves, units);
+  const GrLaunch shape = gr_launch_shape(M, N, parts, col_tiles, glu, waves, units, cols);
+  PYLON_REQUIRE(cols >= 0 && cols <= shape.waves * (glu ? 1 : col_tiles) * 16,
+                "gemm_rows: %d columns per workgroup are more than the tiles of its %d waves hold", cols, shape.waves);
 #define GO(MT)                                                                                              \
   do {                                                                                                      \
     if (glu) launch_rows<MT, 2, true>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, stream); \

@@ -37,8 +37,8 @@ _SIGNATURES = {
     "pylon_attention_prefill": [P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, P],
     "pylon_gemm_tiled": [P, I, P, I, P, I, I, I, I, L, L, L, P],
     "pylon_gemm_skinny": [P, I, P, P, I, I, I, L, L, L, I, L, I, P],
-    "pylon_gemm_rows": [P, I, P, P, I, I, I, L, L, L, I, L, I, I, I, P],
-    "pylon_gemm_rows_shape": [I, L, I, I, I, I, I, P],
+    "pylon_gemm_rows": [P, I, P, P, I, I, I, L, L, L, I, L, I, I, I, I, P],
+    "pylon_gemm_rows_shape": [I, I, I, I, I, I, I, I, P],
     "pylon_argmax": [P, P, I, I, L, P, P, P, L, P],
     "pylon_argmax_static": [P, P, I, I, L, P, P, P],
     "pylon_probe_read": [P, L, P, P],

@@ -494,15 +494,17 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype
 
 
 def gemm_rows(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype = torch.bfloat16,
-              parts: int = 1, col_tiles: int = 1, glu: bool = False, waves: int = 0,
+              parts: int = 1, col_tiles: int = 1, glu: bool = False, waves: int = 0, cols: int = 0,
               out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``x @ weight.T`` for at most 64 rows of bfloat16 ``x``, made for 17 to 64: the rows of
-    ``x`` pass through LDS once per workgroup of 64 (``col_tiles=1``) or 128 (``col_tiles=2``)
-    columns and ``weight`` is streamed once.  ``parts > 1`` cuts K into that many ranges and
-    returns float32 partial results ``[parts, M, N]`` for the consumer to add.  ``glu``:
-    ``weight`` is a fused ``[2N, K]`` gate/up matrix and the result is
-    ``silu(x @ gate.T) * (x @ up.T)``, rounded once.  ``waves``: wavefronts per workgroup,
-    4 or 2 (0: the kernel's choice); the sums do not depend on it."""
+    """``x @ weight.T`` for at most 64 rows of bfloat16 ``x``: the rows of ``x`` pass through
+    LDS once per workgroup of up to 64 (``col_tiles=1``) or 128 (``col_tiles=2``) columns and
+    ``weight`` is streamed once.  ``parts > 1`` cuts K into that many ranges and returns
+    float32 partial results ``[parts, M, N]`` for the consumer to add.  ``glu``: ``weight`` is
+    a fused ``[2N, K]`` gate/up matrix and the result is ``silu(x @ gate.T) * (x @ up.T)``,
+    rounded once.  ``waves``: wavefronts per workgroup, 4 or 2 (0: the kernel's choice);
+    ``cols``: columns per workgroup (0: the kernel's choice, an equal share for every
+    workgroup of whole rounds over the compute units where that pays).  The sums depend on
+    neither."""
     if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
         raise KernelError(f"gemm_rows: cannot multiply {tuple(x.shape)} by the transpose of {tuple(weight.shape)}")
     m, k = x.shape
@@ -523,7 +525,7 @@ def gemm_rows(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype =
         raise KernelError(f"gemm_rows: out must be contiguous, on the GPU and of shape {shape}")
     _lib.call("pylon_gemm_rows", out.data_ptr(), dtype_code(out.dtype), x.data_ptr(), weight.data_ptr(),
               m, n, k, x.stride(0), weight.stride(0), n, parts, m * n, int(col_tiles), 1 if glu else 0, int(waves),
-              _stream())
+              int(cols), _stream())
     return out
 
 

@@ -43,7 +43,9 @@ def rows_split(n: int, k: int, rows: int = STREAM_ROWS, units: int = UNITS) -> t
     Workgroups of 128 columns for deep matrices (beyond 16 rows, where the rows of x weigh
     more, from a depth of 8192) and for wide ones, else of 64; K cut into the largest power of
     two of parts (at most 16, of at least 256 elements each) that keeps the workgroups at one
-    per compute unit or fewer: more of them only re-read the rows of x."""
+    per compute unit or fewer: more of them only re-read the rows of x.  (The kernel then gives
+    every workgroup the same share of the columns, so that the launch fills whole rounds of the
+    units, where the share stays at least as many rows of w as there are rows of x.)"""
     col_tiles = 2 if (k >= 8192 and rows > FEW_ROWS) or k >= 16384 or n > 4096 else 1
     groups = -(-n // (64 * col_tiles))
     parts = 1

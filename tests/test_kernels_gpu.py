@@ -242,7 +242,8 @@ def test_gemm_skinny(ops, shape):
 def test_gemm_rows_at_random_shapes(ops):
     """Sixty seeded draws of every argument (rows 1 to 64, 1 to 700 columns, depths that are
     multiples of 8 up to 1,496, parts beyond the number of chunks, both widths and wave
-    counts, the gated form) against a float64 product."""
+    counts, the gated form) against a float64 product; and with any number of columns per
+    workgroup, down to one, the bits of the kernel's own choice."""
     rng = np.random.default_rng(2024)
     for case in range(60):
         m = int(rng.integers(1, 65))
@@ -258,6 +259,10 @@ def test_gemm_rows_at_random_shapes(ops):
             want = g / (1 + np.exp(-g)) * u
         got = ops.gemm_rows(a.to(DEV), w.to(DEV), out_dtype=torch.float32, parts=parts, col_tiles=col_tiles,
                             glu=glu, waves=waves)
+        cols = int(rng.integers(1, 2 * (16 if glu else 16 * col_tiles) + 1))  # what two waves hold at most
+        shared = ops.gemm_rows(a.to(DEV), w.to(DEV), out_dtype=torch.float32, parts=parts, col_tiles=col_tiles,
+                               glu=glu, waves=waves, cols=cols)
+        assert torch.equal(shared, got), (case, m, n, k, parts, col_tiles, glu, waves, cols)
         got = f64(got).sum(0) if parts > 1 else f64(got)
         assert got.shape == want.shape, (case, m, n, k)
         assert np.abs(got - want).max() <= tol(torch.float32, max(np.abs(want).max(), 1e-3)), \

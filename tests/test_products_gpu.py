@@ -7,32 +7,30 @@ The vocabulary head is /root/reference/src/pylon/model/model.py:140-144, q/k/v a
 projection /root/reference/src/pylon/model/layers.py:126,138, gate/up and down :26-27.
 
 Kernel instance reached per case (``gemm_rows_kernel<MT, CT, GLU, WAVES, TO>`` with MT =
-ceil(rows / 16); "spread": the waves of a workgroup take column groups one per compute unit
-apart; ``groups x parts`` workgroups):
+ceil(rows / 16); ``groups x parts`` workgroups of ``c`` columns each: every workgroup of a
+launch gets the same share of the columns, a whole number of rounds over the 256 compute
+units, unless that would make it re-read more rows of x than it streams rows of w):
 
-=========  =====================  ======================================  ===================
-product    1, 8, 16 rows          17, 48, 64 rows                         65, 130 rows
-=========  =====================  ======================================  ===================
-4b qkv     rows CT1 2 waves,      library, bfloat16                       library, bfloat16
-           256x1 spread
-4b out     rows CT1 4w 40x4       rows CT1 4w 40x4                        library, bfloat16
-4b gate/up rows GLU 4w 256x1      rows GLU 4w 256x1 spread                library + silu_gate
-           spread
-4b down    rows CT1 4w 40x4       rows CT2 4w 20x8                        library, bfloat16
-4b head    rows CT2 4w 1187x1     rows CT2 4w 1187x1                      library, float32
-8b qkv     rows CT1 2w 256x1      library                                 library
-           spread
-8b out     rows CT1 4w 64x4       rows CT1 4w 64x4                        library
-8b gate/up skinny GLU             rows GLU 4w 256x1 spread                library + silu_gate
-8b down    rows CT1 4w 64x4       rows CT2 4w 32x8                        library
-8b head    skinny                 rows CT2 4w 1187x1                      library, float32
-32b qkv    rows CT1 4w 256x1      library                                 library
-           spread
-32b out    rows CT2 4w 40x4       library, float32                        library
-32b g/u    rows GLU 4w 400x1      library float32 + silu_gate             library + silu_gate
-32b down   rows CT2 4w 40x4       rows CT2 4w 40x4                        library
-32b head   rows CT2 4w 1187x1     rows CT2 4w 1187x1                      library, float32
-=========  =====================  ======================================  ===================
+=========  ========================  =====================================  ===================
+product    1, 8, 16 rows             17, 48, 64 rows                        65, 130 rows
+=========  ========================  =====================================  ===================
+4b qkv     rows CT1 2w 256x1 c24     library, bfloat16                      library, bfloat16
+4b out     rows CT1 4w 64x4 c40      rows CT1 4w 64x4 c40 at 17 rows,       library, bfloat16
+                                     40x4 c64 at 48 and 64
+4b gate/up rows GLU 4w 256x1 c38     rows GLU 4w 256x1 c38                  library + silu_gate
+4b down    rows CT1 4w 64x4 c40      rows CT2 4w 32x8 c80                   library, bfloat16
+4b head    rows CT2 4w 1277x1 c119   rows CT2 4w 1187x1 c128                library, float32
+8b qkv     rows CT1 2w 256x1 c24     library                                library
+8b out     rows CT1 4w 64x4 c64      rows CT1 4w 64x4 c64                   library
+8b gate/up skinny GLU                rows GLU 4w 256x1 c48                  library + silu_gate
+8b down    rows CT1 4w 64x4 c64      rows CT2 4w 32x8 c128                  library
+8b head    skinny                    rows CT2 4w 1187x1 c128                library, float32
+32b qkv    rows CT1 4w 256x1 c40     library                                library
+32b out    rows CT2 4w 64x4 c80      library, float32                       library
+32b g/u    rows GLU 4w 512x1 c50     library float32 + silu_gate            library + silu_gate
+32b down   rows CT2 4w 64x4 c80      rows CT2 4w 64x4 c80                   library
+32b head   rows CT2 4w 1277x1 c119   rows CT2 4w 1187x1 c128                library, float32
+=========  ========================  =====================================  ===================
 """
 import ctypes
 import zlib
@@ -49,24 +47,26 @@ VOCAB = 151936
 SIZES = {"4b": (2560, 4096, 1024, 9728), "8b": (4096, 4096, 1024, 12288), "32b": (5120, 8192, 1024, 25600)}
 ROWS = (1, 8, 16, 17, 48, 64, 65, 130)
 
-# (kernel, parts, col_tiles, (waves, groups, spread)) for few (<= 16) and many (17..64) rows
+# (kernel, parts, col_tiles, (waves, groups, columns per workgroup)) for few (<= 16) and many
+# (17..64) rows; a dict where the many differ among themselves
 R = "rows"
 EXPECT = {
-    ("4b", "qkv"): ((R, 1, 1, (2, 256, 1)), ("library",)),
-    ("4b", "out"): ((R, 4, 1, (4, 40, 0)), (R, 4, 1, (4, 40, 0))),
-    ("4b", "gate_up"): ((R, 1, 2, (4, 256, 1)), (R, 1, 2, (4, 256, 1))),
-    ("4b", "down"): ((R, 4, 1, (4, 40, 0)), (R, 8, 2, (4, 20, 0))),
-    ("4b", "head"): ((R, 1, 2, (4, 1187, 0)), (R, 1, 2, (4, 1187, 0))),
-    ("8b", "qkv"): ((R, 1, 1, (2, 256, 1)), ("library",)),
-    ("8b", "out"): ((R, 4, 1, (4, 64, 0)), (R, 4, 1, (4, 64, 0))),
-    ("8b", "gate_up"): (("skinny",), (R, 1, 2, (4, 256, 1))),
-    ("8b", "down"): ((R, 4, 1, (4, 64, 0)), (R, 8, 2, (4, 32, 0))),
-    ("8b", "head"): (("skinny",), (R, 1, 2, (4, 1187, 0))),
-    ("32b", "qkv"): ((R, 1, 1, (4, 256, 1)), ("library",)),
-    ("32b", "out"): ((R, 4, 2, (4, 40, 0)), ("library",)),
-    ("32b", "gate_up"): ((R, 1, 2, (4, 400, 0)), ("library",)),
-    ("32b", "down"): ((R, 4, 2, (4, 40, 0)), (R, 4, 2, (4, 40, 0))),
-    ("32b", "head"): ((R, 1, 2, (4, 1187, 0)), (R, 1, 2, (4, 1187, 0))),
+    ("4b", "qkv"): ((R, 1, 1, (2, 256, 24)), ("library",)),
+    ("4b", "out"): ((R, 4, 1, (4, 64, 40)), {17: (R, 4, 1, (4, 64, 40)), 48: (R, 4, 1, (4, 40, 64)),
+                                             64: (R, 4, 1, (4, 40, 64))}),
+    ("4b", "gate_up"): ((R, 1, 2, (4, 256, 38)), (R, 1, 2, (4, 256, 38))),
+    ("4b", "down"): ((R, 4, 1, (4, 64, 40)), (R, 8, 2, (4, 32, 80))),
+    ("4b", "head"): ((R, 1, 2, (4, 1277, 119)), (R, 1, 2, (4, 1187, 128))),
+    ("8b", "qkv"): ((R, 1, 1, (2, 256, 24)), ("library",)),
+    ("8b", "out"): ((R, 4, 1, (4, 64, 64)), (R, 4, 1, (4, 64, 64))),
+    ("8b", "gate_up"): (("skinny",), (R, 1, 2, (4, 256, 48))),
+    ("8b", "down"): ((R, 4, 1, (4, 64, 64)), (R, 8, 2, (4, 32, 128))),
+    ("8b", "head"): (("skinny",), (R, 1, 2, (4, 1187, 128))),
+    ("32b", "qkv"): ((R, 1, 1, (4, 256, 40)), ("library",)),
+    ("32b", "out"): ((R, 4, 2, (4, 64, 80)), ("library",)),
+    ("32b", "gate_up"): ((R, 1, 2, (4, 512, 50)), ("library",)),
+    ("32b", "down"): ((R, 4, 2, (4, 64, 80)), (R, 4, 2, (4, 64, 80))),
+    ("32b", "head"): ((R, 1, 2, (4, 1277, 119)), (R, 1, 2, (4, 1187, 128))),
 }
 
 
@@ -86,11 +86,11 @@ def shape_of(model: str, product: str):
             "down": (hidden, inter), "head": (VOCAB, hidden)}[product]
 
 
-def launch_shape(n, ldw, parts, col_tiles, glu):
+def launch_shape(rows, n, parts, col_tiles, glu, units=0):
     from pylon_amd.kernels import library
 
     out = (ctypes.c_int * 3)()
-    assert library.load().pylon_gemm_rows_shape(n, ldw, parts, col_tiles, glu, 0, 0, out) == 0
+    assert library.load().pylon_gemm_rows_shape(rows, n, parts, col_tiles, glu, 0, units, 0, out) == 0
     return tuple(out)
 
 
@@ -108,7 +108,7 @@ def chosen(model, product, rows, units):
     if c.kernel != "rows":
         return (c.kernel,)
     glu = product == "gate_up"
-    return (c.kernel, c.parts, c.col_tiles, launch_shape(n // 2 if glu else n, k, c.parts, c.col_tiles, int(glu)))
+    return (c.kernel, c.parts, c.col_tiles, launch_shape(rows, n // 2 if glu else n, c.parts, c.col_tiles, int(glu)))
 
 
 @pytest.mark.parametrize("product", ["qkv", "out", "gate_up", "down", "head"])
@@ -131,7 +131,8 @@ def test_a_product_at_its_real_size(ops, model, product):
     assert units == 256  # the expectations above are those of an MI355X
     for rows in ROWS:
         if rows <= 64:
-            assert chosen(model, product, rows, units) == (few if rows <= 16 else many), (model, product, rows)
+            expected = few if rows <= 16 else (many[rows] if isinstance(many, dict) else many)
+            assert chosen(model, product, rows, units) == expected, (model, product, rows)
         xr = x[:rows].contiguous()
         if product in ("out", "down"):
             got = ops.linear_for_residual(xr, w, out_dtype=torch.bfloat16)
