@@ -407,12 +407,12 @@ def main() -> int:
             points["mixed_b64_chunk2048_ms"] = round(point["mixed_ms"], 3)
             points["mixed_b64_chunk2048_hbm_frac"] = round(point["bytes"] / (point["mixed_ms"] * 1e-3) / HBM_BYTES_PER_S, 4)
             points["mixed_b64_chunk2048_flops_frac"] = round(chunk_flops / (point["mixed_ms"] * 1e-3) / PEAK_FLOPS[dtype_key], 4)
-            # one prompt of 8,191 tokens (the context's 8,192 less the token it produces), four portions
+            # one prompt as long as the context allows (8,191 tokens: 8,192 less the token it produces), in portions
             long_prompt = context_length - 1
             seconds = prefill_run(runner, cfg, args, long_prompt, repeats=3, seed=14)
             flops = linear_flops_per_token(cfg) * long_prompt + attention_flops(cfg, long_prompt)
-            points["prefill_8191"] = round(long_prompt / seconds, 1)
-            points["prefill_8191_flops_frac"] = round(flops / seconds / PEAK_FLOPS[dtype_key], 4)
+            points[f"prefill_{long_prompt}"] = round(long_prompt / seconds, 1)
+            points[f"prefill_{long_prompt}_flops_frac"] = round(flops / seconds / PEAK_FLOPS[dtype_key], 4)
         rate, first_ms = engine_run(runner, cfg, args, batch=8, seed=9, prompt_len=prompt_len)
         points["engine_b8"], points["engine_b8_first_token_ms"] = round(rate, 1), round(first_ms, 2)
         # the reference's other published workload: 2,048-token prompts, 32 new tokens, 8 at a time
