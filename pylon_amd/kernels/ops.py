@@ -25,7 +25,15 @@ def dtype_code(dtype: torch.dtype) -> int:
         raise KernelError(f"the kernels take float32 and bfloat16, not {dtype}") from None
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream() -> int:
+    """The current stream's handle.  A step asks for it once per launch, a few hundred times:
+    the two raw calls take a fifth of a microsecond, ``torch.cuda.current_stream()`` six."""
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
     return torch.cuda.current_stream().cuda_stream
 
 
