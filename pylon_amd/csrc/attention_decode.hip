@@ -38,9 +38,14 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 // What the kernel needs to prepare q, k and v itself (PREP): the raw projection
 // [tokens, row_stride] with q heads first, then k heads, then v heads.
+// With n_parts > 0 the projection comes as that many float partial sums (a product whose K
+// was cut over workgroups), part_stride elements apart; the kernel adds them in order and
+// rounds the sum to bfloat16 once, which is what a projection stored as bfloat16 holds.
 struct DecodePrep {
-  const uint16_t* qkv;
+  const void* qkv;
   long long row_stride;
+  int n_parts;
+  long long part_stride;
   const float* q_weight;  // per-head RMSNorm weights, or null
   const float* k_weight;
   float eps;
@@ -66,7 +71,9 @@ static __host__ __device__ size_t decode_lds_floats(int n_waves, int gp, int hea
 }
 
 // EPL = head_dim / 64, KSTEPS = head_dim / 32, GP = heads per group rounded up to 1, 2, 4, 8, 16
-template <int EPL, int KSTEPS, int GP, bool PREP>
+// PARTS (with PREP): the projection comes as float partial sums (an instance of its own, so
+// that the others keep their registers).
+template <int EPL, int KSTEPS, int GP, bool PREP, bool PARTS = false>
 __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, typename DecodeCache<PREP>::ptr k_cache,
     typename DecodeCache<PREP>::ptr v_cache, const int* __restrict__ block_table, int table_width,
@@ -123,21 +130,26 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
     constexpr int LPH = HD / 8, HPW = PYLON_WAVE / LPH;
     // the token's rotation table, one private copy per wave: no workgroup barrier before use
     float* cs = reinterpret_cast<float*>(q_lds + GP * HD) + wave * HD;
-    const uint16_t* row = prep.qkv + static_cast<size_t>(t) * prep.row_stride;
+    const size_t row_at = static_cast<size_t>(t) * prep.row_stride;
     // the new key and value are stored by the one workgroup whose keys include them
     const int slot = (prep.slot_map != nullptr && holds_last) ? prep.slot_map[t] : -1;
     const int jobs = group + (slot >= 0 ? 2 : 0);
     stored_new = slot >= 0;
     const int j = lane % LPH;
     // job -> where its head lies in the projection's row
-    auto source = [&](int job) {
+    auto load = [&](int job, float v[8]) {
       const int head = job < group ? kvh * group + job : n_heads + (job == group ? 0 : n_kv_heads) + kvh;
-      return row + static_cast<size_t>(head) * HD + 8 * j;
+      const size_t at = row_at + static_cast<size_t>(head) * HD + 8 * j;
+      if constexpr (PARTS) {
+        sum8_parts(static_cast<const float*>(prep.qkv) + at, prep.n_parts, prep.part_stride, v);
+      } else {
+        load8_bf16(static_cast<const uint16_t*>(prep.qkv) + at, v);
+      }
     };
     // The first round's loads do not wait for the position.
     int job = wave * HPW + lane / LPH;
     float v[8];
-    load8_bf16(source(job < jobs ? job : jobs - 1), v);
+    load(job < jobs ? job : jobs - 1, v);
     if (prep.inv_freq != nullptr && wave * HPW < jobs) {
       const float fpos = static_cast<float>(pos);
       for (int i = lane; i < HD / 2; i += PYLON_WAVE) {
@@ -151,7 +163,7 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
       job = h0 + lane / LPH;
       const bool valid = job < jobs;
       if (!valid) job = jobs - 1;
-      if (h0 != wave * HPW) load8_bf16(source(job), v);
+      if (h0 != wave * HPW) load(job, v);
       const bool is_q = job < group, is_key = job == group;
       const float* weight = is_q ? prep.q_weight : (is_key ? prep.k_weight : nullptr);
       norm_rotate8<HD>(v, j, weight, prep.eps, (prep.inv_freq != nullptr && (is_q || is_key)) ? cs : nullptr);
@@ -401,7 +413,7 @@ static size_t decode_lds_bytes(int n_waves, int gp, int head_dim, bool prep) {
                : 0);
 }
 
-template <int EPL, bool PREP>
+template <int EPL, bool PREP, bool PARTS = false>
 static int launch_decode(void* out, const void* q, void* k_cache, void* v_cache,
                          const int* block_table, int table_width, const int* tok_row,
                          const int* positions, int tokens, int n_heads, int n_kv_heads, int page_size,
@@ -414,7 +426,7 @@ static int launch_decode(void* out, const void* q, void* k_cache, void* v_cache,
   const size_t lds = decode_lds_bytes(n_waves, gp, EPL * 64, PREP);
   dim3 grid(n_kv_heads, tokens, n_cuts), block(n_waves * PYLON_WAVE);
 #define LAUNCH(GP)                                                                                         \
-  hipLaunchKernelGGL((attention_decode_kernel<EPL, EPL * 2, GP, PREP>), grid, block, lds, stream,          \
+  hipLaunchKernelGGL((attention_decode_kernel<EPL, EPL * 2, GP, PREP, PARTS>), grid, block, lds, stream,   \
                      (uint16_t*)out, (const uint16_t*)q, (typename DecodeCache<PREP>::ptr)k_cache,         \
                      (typename DecodeCache<PREP>::ptr)v_cache, block_table, table_width, tok_row, positions, \
                      n_heads, n_kv_heads, page_size, window, scale, prep, partial)
@@ -492,12 +504,13 @@ extern "C" int pylon_attention_decode(void* out, const void* q, const void* k_ca
 }
 
 // The same from the raw projection qkv: [tokens, row_stride] bf16 with q heads first, then
-// (if slot_map is given) k heads, then v heads.  Each token's key and value are normed,
+// (if slot_map is given) k heads, then v heads; or, with qkv_parts > 0, that many float
+// partial sums of it, part_stride elements apart, which the kernel adds and rounds to bf16.  Each token's key and value are normed,
 // rotated (inv_freq: head_dim/2 frequencies for a rotation of the whole head, or null) and
 // stored at slot_map[t] before the cache is read; a negative slot stores nothing.  With
 // slot_map null only the queries are prepared (a layer that reads another layer's cache).
-extern "C" int pylon_attention_decode_fused(void* out, const void* qkv, long long row_stride,
-                                            const float* q_weight, const float* k_weight, float eps,
+extern "C" int pylon_attention_decode_fused(void* out, const void* qkv, long long row_stride, int qkv_parts,
+                                            long long part_stride, const float* q_weight, const float* k_weight, float eps,
                                             const float* inv_freq, void* k_cache, void* v_cache,
                                             const int* slot_map, const int* block_table, int table_width,
                                             const int* tok_row, const int* positions, int tokens,
@@ -513,11 +526,21 @@ extern "C" int pylon_attention_decode_fused(void* out, const void* qkv, long lon
                 row_stride, heads, head_dim);
   PYLON_REQUIRE(row_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(qkv) & 15) == 0,
                 "attention_decode_fused: the projection's rows must be 16-byte aligned");
+  PYLON_REQUIRE(qkv_parts >= 0 && qkv_parts <= 64, "attention_decode_fused: 0 to 64 partial sums, got %d", qkv_parts);
+  PYLON_REQUIRE(qkv_parts == 0 || (part_stride % 4 == 0 && part_stride >= static_cast<long long>(tokens - 1) * row_stride + heads * head_dim),
+                "attention_decode_fused: the partial sums overlap or are not 16-byte aligned");
   if (tokens == 0) return 0;
-  const DecodePrep prep = {static_cast<const uint16_t*>(qkv), row_stride, q_weight, k_weight, eps, inv_freq, slot_map};
+  const DecodePrep prep = {qkv, row_stride, qkv_parts, part_stride, q_weight, k_weight, eps, inv_freq, slot_map};
 #define GO(D)                                                                                            \
-  launch_decode<D, true>(out, nullptr, k_cache, v_cache, block_table, table_width, tok_row, positions, tokens, \
-                         n_heads, n_kv_heads, page_size, window, scale, n_waves, prep, n_cuts, partial, stream)
+  do {                                                                                                   \
+    if (qkv_parts > 0)                                                                                   \
+      launch_decode<D, true, true>(out, nullptr, k_cache, v_cache, block_table, table_width, tok_row, positions, \
+                                   tokens, n_heads, n_kv_heads, page_size, window, scale, n_waves, prep, n_cuts, \
+                                   partial, stream);                                                     \
+    else                                                                                                 \
+      launch_decode<D, true>(out, nullptr, k_cache, v_cache, block_table, table_width, tok_row, positions, tokens, \
+                             n_heads, n_kv_heads, page_size, window, scale, n_waves, prep, n_cuts, partial, stream); \
+  } while (0)
   switch (head_dim / 64) {
     case 1: GO(1); break;
     case 2: GO(2); break;

@@ -86,6 +86,41 @@ __device__ __forceinline__ void load8_bf16(const uint16_t* __restrict__ src, flo
   }
 }
 
+// v = the sum of n_parts float vectors of 8 (32-byte aligned), stride elements apart, added in
+// order and rounded to bfloat16 once.  For the usual counts every load is issued before the
+// first addition.
+__device__ __forceinline__ void sum8_parts(const float* __restrict__ src, int n_parts, long long stride, float v[8]) {
+  auto take = [&](int p, float4& a, float4& b) {
+    const float4* at = reinterpret_cast<const float4*>(src + p * stride);
+    a = at[0], b = at[1];
+  };
+  float4 lo, hi;
+  if (n_parts == 2 || n_parts == 4) {
+    float4 a[4], b[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) take(p < n_parts ? p : 0, a[p], b[p]);
+    lo = a[0], hi = b[0];
+#pragma unroll
+    for (int p = 1; p < 4; ++p) {
+      if (p < n_parts) {
+        lo.x += a[p].x, lo.y += a[p].y, lo.z += a[p].z, lo.w += a[p].w;
+        hi.x += b[p].x, hi.y += b[p].y, hi.z += b[p].z, hi.w += b[p].w;
+      }
+    }
+  } else {
+    take(0, lo, hi);
+    for (int p = 1; p < n_parts; ++p) {
+      float4 a, b;
+      take(p, a, b);
+      lo.x += a.x, lo.y += a.y, lo.z += a.z, lo.w += a.w;
+      hi.x += b.x, hi.y += b.y, hi.z += b.z, hi.w += b.w;
+    }
+  }
+  const float sums[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = __uint_as_float(static_cast<uint32_t>(float_to_bf16_bits(sums[e])) << 16);
+}
+
 __device__ __forceinline__ void store8_bf16(uint16_t* __restrict__ dst, const float v[8]) {
   uint32_t w[4];
 #pragma unroll

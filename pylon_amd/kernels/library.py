@@ -33,7 +33,7 @@ _SIGNATURES = {
     "pylon_qkv_prepare": [P, P, P, P, I, L, P, P, F, P, I, P, P, I, I, I, I, I, P],
     "pylon_paged_attention": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, P],
     "pylon_attention_decode": [P, P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, L, P],
-    "pylon_attention_decode_fused": [P, P, L, P, P, F, P, P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, L, P],
+    "pylon_attention_decode_fused": [P, P, L, I, L, P, P, F, P, P, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, L, P],
     "pylon_attention_prefill": [P, P, P, P, P, I, P, I, I, I, I, I, I, F, I, P],
     "pylon_gemm_tiled": [P, I, P, I, P, I, I, I, I, L, L, L, P],
     "pylon_gemm_skinny": [P, I, P, P, I, I, I, L, L, L, I, L, I, P],

@@ -322,15 +322,14 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     return out
 
 
-def decode_fused_ok(qkv: torch.Tensor, k_cache: torch.Tensor, *, tokens: int, n_heads: int, head_dim: int,
+def decode_fused_ok(qkv_dtype: torch.dtype, k_cache: torch.Tensor, *, tokens: int, n_heads: int, head_dim: int,
                     rot_dim: int) -> bool:
-    """Whether the decode kernel can prepare q, k and v itself: its geometry, and a rotation
-    of the whole head or none."""
+    """Whether the decode kernel can prepare q, k and v itself from a projection of
+    ``qkv_dtype``: its geometry, and a rotation of the whole head or none."""
     n_kv_heads = k_cache.shape[2]
-    return (qkv.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and head_dim in DECODE_HEAD_DIMS
+    return (qkv_dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and head_dim in DECODE_HEAD_DIMS
             and tokens <= DECODE_MAX_TOKENS and n_heads % n_kv_heads == 0 and n_heads // n_kv_heads <= 16
-            and rot_dim in (0, head_dim) and qkv.stride(0) % 8 == 0 and qkv.stride(1) == 1
-            and qkv.data_ptr() % 16 == 0)
+            and rot_dim in (0, head_dim))
 
 
 def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -341,13 +340,24 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
                            n_cuts: int = 1) -> torch.Tensor:
     """:func:`qkv_prepare` and :func:`attention_decode` in one launch: from the raw projection
     ``qkv`` ``[tokens, (n_heads + 2 kv_heads) * head_dim]`` (``[tokens, n_heads * head_dim]``
-    when ``slot_map`` is None and nothing is stored).  Returns ``[tokens, n_heads, head_dim]``."""
+    when ``slot_map`` is None and nothing is stored), bfloat16, or from float32 partial sums
+    ``[parts, tokens, width]`` of it, which the kernel adds in order and rounds to bfloat16
+    once.  Returns ``[tokens, n_heads, head_dim]``."""
     pages, psize, n_kv_heads, head_dim = k_cache.shape
-    tokens = qkv.shape[0]
     store = slot_map is not None
-    if qkv.dim() != 2 or qkv.shape[1] != (n_heads + (2 * n_kv_heads if store else 0)) * head_dim:
+    parts = 0
+    if qkv.dim() == 3:
+        if qkv.dtype != torch.float32 or not qkv.is_contiguous():
+            raise KernelError("attention_decode_fused: partial sums come as a contiguous float32 stack")
+        parts = qkv.shape[0]
+    elif qkv.dim() != 2 or qkv.dtype != torch.bfloat16:
+        raise KernelError("attention_decode_fused takes a bfloat16 projection or float32 partial sums of it")
+    tokens, width = qkv.shape[-2:]
+    if width != (n_heads + (2 * n_kv_heads if store else 0)) * head_dim:
         raise KernelError("attention_decode_fused: the projection's width does not match the heads")
-    if not decode_fused_ok(qkv, k_cache, tokens=tokens, n_heads=n_heads, head_dim=head_dim,
+    if qkv.stride(-1) != 1 or qkv.stride(-2) % 8 or qkv.data_ptr() % 16:
+        raise KernelError("attention_decode_fused: the projection's rows must be contiguous and 16-byte aligned")
+    if not decode_fused_ok(torch.bfloat16, k_cache, tokens=tokens, n_heads=n_heads, head_dim=head_dim,
                            rot_dim=0 if inv_freq is None else 2 * inv_freq.numel()):
         raise KernelError("attention_decode_fused does not take this geometry")
     if psize != page_size or k_cache.shape != v_cache.shape or v_cache.dtype != k_cache.dtype:
@@ -364,9 +374,10 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
             raise KernelError("attention_decode_fused: without row ids the table needs a row per token")
     elif tok_row.numel() != tokens:
         raise KernelError("attention_decode_fused: one row id per token is required")
-    out = torch.empty((tokens, n_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+    out = torch.empty((tokens, n_heads, head_dim), dtype=torch.bfloat16, device=qkv.device)
     scratch = _decode_scratch(tokens, n_heads, head_dim, n_cuts, qkv.device)
-    _lib.call("pylon_attention_decode_fused", _dev(out, "out"), qkv.data_ptr(), qkv.stride(0),
+    _lib.call("pylon_attention_decode_fused", _dev(out, "out"), qkv.data_ptr(), qkv.stride(-2), parts,
+              qkv.stride(0) if parts else 0,
               _dev(q_weight, "q_weight", torch.float32), _dev(k_weight, "k_weight", torch.float32), float(eps),
               _dev(inv_freq, "inv_freq", torch.float32), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
               _dev(slot_map, "slot_map", torch.int32), _dev(block_table, "block_table", torch.int32),
@@ -573,6 +584,18 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.d
         y = y if out_dtype == torch.bfloat16 else y.to(out_dtype)
         return y if out is None else out.copy_(y)
     return gemm_tiled(x, weight, out_dtype=out_dtype, out=out)
+
+
+def linear_summed_later(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:
+    """``x @ weight.T`` for a consumer that takes either the product in ``out_dtype`` or float32
+    partial sums ``[parts, M, N]`` of it, to be added in order and rounded to ``out_dtype`` once
+    (:func:`attention_decode_fused` does): from 17 to 64 bfloat16 rows the weight-streaming
+    kernel with K cut over workgroups (:func:`plan.plan_summed_later`), else :func:`linear`."""
+    if out_dtype == torch.bfloat16 and _streaming_ok(x, weight, STREAM_ROWS):
+        choice = plan.plan_summed_later(x.shape[0], *weight.shape, units=_lib.compute_units())
+        if choice.kernel == "rows" and choice.parts > 1:
+            return gemm_rows(x, weight, out_dtype=torch.float32, parts=choice.parts, col_tiles=choice.col_tiles)
+    return linear(x, weight, out_dtype=out_dtype)
 
 
 def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:

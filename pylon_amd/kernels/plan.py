@@ -105,6 +105,21 @@ def plan_projection(rows: int, n: int, k: int) -> Product:
     return Product("rows") if few else Product("library")
 
 
+def plan_summed_later(rows: int, n: int, k: int, units: int = UNITS) -> Product:
+    """A projection whose consumer can add float partial sums itself (q/k/v in front of the
+    decode attention that prepares its own operands).  Beyond 16 rows the rows kernel with K
+    cut over workgroups then beats the library, which does not cut K: 6144 x 2560 at 17, 32,
+    48 and 64 rows 9.0, 9.5, 10.8 and 11.7 us (four parts of 128 columns) against 11.0, 11.8,
+    15.3 and 15.5; 6144 x 4096 11.8 to 14.9 against 14.5 to 17.9; 10240 x 5120 (two parts)
+    21.5 to 28.1 against 24.4 to 32.8.  Without a cut, and up to 16 rows, as
+    :func:`plan_projection`."""
+    if FEW_ROWS < rows <= STREAM_ROWS and n < TALL:
+        parts, col_tiles = rows_split(n, k, rows, units)
+        if parts > 1:
+            return Product("rows", parts, col_tiles)
+    return plan_projection(rows, n, k)
+
+
 def plan_gated(rows: int, n_half: int, k: int, row_stride: int) -> Product:
     """``silu(x gate^T) * (x up^T)`` over a fused matrix of ``2 * n_half`` rows, ``rows`` <= 64;
     "library" means its float32 result followed by the activation kernel.

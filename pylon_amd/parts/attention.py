@@ -58,12 +58,13 @@ class Attention(Part):
         weight = self.params["qkv"]
         if not stores:
             weight = weight[: spec.q_size]
-        qkv = ops.linear(h, weight, out_dtype=self.dtype)
         rotary = self.position.rotary()
         if ctx.decode_only and cache.k is not None and ops.decode_fused_ok(
-                qkv, cache.k, tokens=tokens, n_heads=spec.n_heads, head_dim=spec.head_dim,
+                self.dtype, cache.k, tokens=tokens, n_heads=spec.n_heads, head_dim=spec.head_dim,
                 rot_dim=rotary[1] if rotary else 0):
-            # one launch norms and rotates q and k, stores k and v, and attends
+            # one launch adds the projection's partial sums if it comes as such, norms and
+            # rotates q and k, stores k and v, and attends
+            qkv = ops.linear_summed_later(h, weight, out_dtype=self.dtype)
             cuts, splits = ops.decode_launch(tokens, spec.n_kv_heads, self._span(ctx))
             context = ops.attention_decode_fused(
                 qkv, cache.k, cache.v, cache.block_table, None, ctx.positions,
@@ -74,6 +75,7 @@ class Attention(Part):
             )
             return ops.linear_for_residual(context.view(tokens, spec.q_size), self.params["out"],
                                            out_dtype=self.dtype)
+        qkv = ops.linear(h, weight, out_dtype=self.dtype)
         q = torch.empty((tokens, spec.n_heads, spec.head_dim), dtype=self.dtype, device=h.device)
         ops.qkv_prepare(
             qkv, q, cache.k, cache.v,

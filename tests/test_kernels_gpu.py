@@ -805,6 +805,22 @@ def test_decode_attention_that_prepares_q_k_v_itself(ops, geom, store):
                 window=window, scale=hd ** -0.5, n_splits=splits, n_cuts=cuts)
             assert torch.equal(got, want), (window, splits, cuts)
             assert torch.equal(kc2, kc) and torch.equal(vc2, vc)
+    # The projection as float partial sums (a product whose K was cut over workgroups): added in
+    # order and rounded to bfloat16 once, they give the bits of the projection so rounded.
+    for parts in (2, 3, 4, 7):
+        stack = rnd((parts, tokens, width), 60 + parts).to(DEV)
+        total = stack[0].clone()
+        for p in range(1, parts):
+            total = total + stack[p]
+        rounded = total.to(torch.bfloat16)
+        kc3, vc3, kc4, vc4 = kc.clone(), vc.clone(), kc.clone(), vc.clone()
+        common = dict(n_heads=nh, q_weight=qw, k_weight=kw, eps=eps, inv_freq=inv_freq,
+                      slot_map=slots.to(DEV) if store else None, page_size=page, window=None, scale=hd ** -0.5,
+                      n_splits=4, n_cuts=2)
+        want = ops.attention_decode_fused(rounded, kc3, vc3, table.to(DEV), None, positions.to(DEV), **common)
+        got = ops.attention_decode_fused(stack, kc4, vc4, table.to(DEV), None, positions.to(DEV), **common)
+        assert torch.equal(got, want), parts
+        assert torch.equal(kc4, kc3) and torch.equal(vc4, vc3), parts
 
 
 def test_kernels_refuse_what_they_cannot_do(ops):

@@ -76,3 +76,20 @@ def test_parts_are_powers_of_two_and_independent_of_the_row_count_within_a_class
         assert len(few) == 1 and len(many) == 1  # one order of additions per class of row counts
         for parts, col_tiles in few | many:
             assert parts & (parts - 1) == 0 and col_tiles in (1, 2)
+
+
+def test_a_projection_whose_consumer_adds_partial_sums_is_cut_over_k_from_17_rows():
+    """q/k/v in front of the decode attention that prepares its own operands: up to 16 rows and
+    for a matrix that is not cut as `plan_projection`; from 17 to 64 rows the rows kernel with
+    K cut (4B and 8B: four parts of 128 columns; 32B: two)."""
+    for name, want in (("4b", (4, 2)), ("8b", (4, 2)), ("32b", (2, 2))):
+        hidden, q, kv, _ = SIZES[name]
+        n = q + 2 * kv
+        for rows in (1, 8, 16):
+            assert plan.plan_summed_later(rows, n, hidden) == plan.plan_projection(rows, n, hidden)
+        for rows in (17, 40, 64):
+            c = plan.plan_summed_later(rows, n, hidden)
+            assert (c.kernel, c.parts, c.col_tiles) == ("rows", *want), (name, rows, c)
+    # a head is never cut (nothing behind it adds), nor is a matrix with too little K per part
+    assert plan.plan_summed_later(40, VOCAB, 2560) == plan.plan_projection(40, VOCAB, 2560)
+    assert plan.plan_summed_later(40, 6144, 256).parts == 1

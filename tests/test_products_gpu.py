@@ -31,6 +31,10 @@ product    1, 8, 16 rows             17, 48, 64 rows                        65, 
 32b down   rows CT2 4w 64x4 c80      rows CT2 4w 64x4 c80                   library
 32b head   rows CT2 4w 1277x1 c119   rows CT2 4w 1187x1 c128                library, float32
 =========  ========================  =====================================  ===================
+
+In front of the decode attention that prepares its own operands q/k/v may also come as float
+partial sums (``ops.linear_summed_later``): from 17 to 64 rows then rows CT2 4w 64x4 c96 (4B,
+8B) and 128x2 c80 (32B), else as above.
 """
 import ctypes
 import zlib
@@ -68,6 +72,10 @@ EXPECT = {
     ("32b", "down"): ((R, 4, 2, (4, 64, 80)), (R, 4, 2, (4, 64, 80))),
     ("32b", "head"): ((R, 1, 2, (4, 1277, 119)), (R, 1, 2, (4, 1187, 128))),
 }
+
+
+# q/k/v for a consumer that adds partial sums, 17..64 rows
+EXPECT_SUMMED = {"4b": (R, 4, 2, (4, 64, 96)), "8b": (R, 4, 2, (4, 64, 96)), "32b": (R, 2, 2, (4, 128, 80))}
 
 
 @pytest.fixture(scope="module")
@@ -149,6 +157,18 @@ def test_a_product_at_its_real_size(ops, model, product):
             assert got.dtype == torch.float32
         else:
             got = ops.linear(xr, w, out_dtype=torch.bfloat16)
+            later = ops.linear_summed_later(xr, w, out_dtype=torch.bfloat16)
+            if 16 < rows <= 64:
+                from pylon_amd.kernels import plan
+
+                c = plan.plan_summed_later(rows, n, k, units=units)
+                assert (c.kernel, c.parts, c.col_tiles, launch_shape(rows, n, c.parts, c.col_tiles, 0)) == \
+                    EXPECT_SUMMED[model], (model, rows)
+                assert later.dtype == torch.float32 and later.shape == (c.parts, rows, n)
+                total = later.sum(0, dtype=torch.float64).cpu().numpy()
+                assert np.abs(total - want[:rows]).max() <= 2e-6 * np.abs(want[:rows]).max(), (model, rows)
+            else:
+                assert torch.equal(later, got)
         ref = want[:rows]
         assert got.shape == ref.shape, (model, product, rows, tuple(got.shape))
         scale = np.abs(ref).max()
