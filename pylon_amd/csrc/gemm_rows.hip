@@ -265,11 +265,12 @@ struct GrLaunch {
 // workgroups than half the units.  cols: columns per workgroup, or 0 for the rule: an equal
 // share for every workgroup of as many whole rounds over the units as workgroups of full
 // width would need (at least 16 columns), unless that makes the workgroups re-read more rows
-// of x than they stream rows of w; then, and beyond 16 rows of x in launches of several rounds,
-// the full width.  Measured at 2560 x 9728, K cut in eight, 32 rows: 13.2 us with 80 columns
+// of x than they stream rows of w; then, and beyond 16 rows of x in launches of several rounds
+// whose last is not mostly empty, the full width.  Measured at 2560 x 9728, K cut in eight, 32 rows: 13.2 us with 80 columns
 // (256 workgroups) against 14.9 with 128 (160); 2560 x 4096 cut in four, 48 rows: 9.15 with
 // 40 columns against 9.08 with 64; the head of 151936 rows at 8 rows of x: 136.5 with 119
-// columns against 141; at 64 rows of x: 181 against 170.5.
+// columns against 141; at 64 rows of x (4.6 rounds): 181 against 170.5; a gate/up matrix of
+// 2 x 17408 rows at 17 rows of x (1.06 rounds of 64 columns): 34 columns in 512 workgroups.
 static GrLaunch gr_launch_shape(int M, int N, int parts, int col_tiles, int glu, int waves, int units, int cols) {
   const int wave_cols = (glu ? 1 : col_tiles) * 16;
   if (waves == 0)
@@ -281,7 +282,9 @@ static GrLaunch gr_launch_shape(int M, int N, int parts, int col_tiles, int glu,
     const long long groups = rounds * units / parts;
     int even = groups > 0 ? static_cast<int>((N + groups - 1) / groups) : full;
     even = even < 16 ? 16 : (even > full ? full : even);
-    const bool pays = M <= 16 || (rounds == 1 && even * (glu ? 2 : 1) >= M);
+    // several rounds of full width are left alone unless the last is mostly empty
+    const bool uneven = rounds == 1 || least * 100 < rounds * units * 85;
+    const bool pays = M <= 16 || (uneven && even * (glu ? 2 : 1) >= M);
     cols = pays ? even : full;
   }
   return GrLaunch{waves, (N + cols - 1) / cols, cols};

@@ -65,26 +65,31 @@ def skinny_parts(n: int, k: int, units: int = UNITS) -> int:
 
 
 def deep_or_narrow(n: int, k: int) -> bool:
-    """Matrices much deeper than wide (a down projection; the library does not cut K) and
-    those of few rows (an out projection): there the rows kernel with K cut into parts beats
-    the library at 17 to 64 rows.  At 64 rows: 2560x4096 9.5 against 14 us, 2560x9728 17
-    against 28, 4096x4096 11 against 15, 4096x12288 24 against 39, 5120x25600 79 against 90;
-    but 5120x8192 30 against 29 and 8192x8192 39 against 35."""
+    """Matrices much deeper than wide (a down projection) and those of few rows (an out
+    projection)."""
     return k >= 2 * n or n <= 4096
 
 
 def plan_residual(rows: int, n: int, k: int, units: int = UNITS) -> Product:
     """A product about to be added to the float32 residual stream (out and down projections),
-    ``rows`` <= 64: float32 sums, never rounded, from whichever kernel.  Up to 16 rows the rows
-    kernel also beats the skinny one (2560x4096 at 8 rows: 6.2 against 8.3 us, 2560x9728 11.5
-    against 13.8, 5120x8192 20 against 23, 5120x25600 52 against 65)."""
+    ``rows`` <= 64: float32 sums, never rounded, from whichever kernel.
+
+    Up to 16 rows the rows kernel beats the skinny one for deep, narrow and moderately wide
+    matrices (2560x4096 at 8 rows: 6.2 against 8.3 us, 2560x9728 11.5 against 13.8, 5120x8192
+    20 against 23, 5120x25600 52 against 65).  From 17 to 64 rows the rows kernel with K cut
+    into parts beats the library, which does not cut K (at 64 rows: 2560x4096 10.0 against
+    14.3 us, 2560x9728 16.0 against 28.0, 4096x4096 11.0 against 15.1, 4096x12288 26.5 against
+    37.5, 5120x5120 16.3 against 21.8, 5120x8192 22.9 against 28.9, 5120x17408 42 against 86,
+    6144x6144 21.5 against 26.8, 10240x10240 48 against 60), except for wide matrices whose rows
+    are of a power-of-two length (8192x8192 36.4 against 33.7, 16384x4096 37.4 against 34.5)."""
     few = rows <= FEW_ROWS
-    if deep_or_narrow(n, k) or (few and n <= 8192):
-        parts, col_tiles = rows_split(n, k, rows, units)
-        return Product("rows", parts, col_tiles)
     if few:
+        if deep_or_narrow(n, k) or n <= 8192:
+            return Product("rows", *rows_split(n, k, rows, units))
         return Product("skinny", skinny_parts(n, k, units))
-    return Product("library")
+    if aliased_rows(k) and n >= 8192:
+        return Product("library")
+    return Product("rows", *rows_split(n, k, rows, units))
 
 
 def plan_projection(rows: int, n: int, k: int) -> Product:
@@ -124,14 +129,17 @@ def plan_gated(rows: int, n_half: int, k: int, row_stride: int) -> Product:
     """``silu(x gate^T) * (x up^T)`` over a fused matrix of ``2 * n_half`` rows, ``rows`` <= 64;
     "library" means its float32 result followed by the activation kernel.
 
-    Against the skinny kernel at 8 rows: 2x9728 x 2560 21 against 25 us, 2x25600 x 5120 98
-    against 109, 2x6144 x 2048 12 against 15; but 2x12288 x 4096 44 against 40 (aliased rows)
-    and 2x3072 x 1024 6.7 against 6.1 (a small matrix).  Against the library and the
-    activation kernel at 64 rows: 27 against 34 us, 48 against 55 (width 4096), 113 against
-    113 (width 5120).  A workgroup of the rows kernel sees its gate rows and, ``n_half`` rows
-    further, its up rows through one descriptor, which spans at most 2 GB."""
+    Against the skinny kernel at 8 rows: 2x9728 x 2560 20 against 25 us, 2x25600 x 5120 90
+    against 105, 2x17408 x 5120 63 against 76, 2x6144 x 2048 13.8 against 15.2; but 2x12288 x
+    4096 44 against 39 (aliased rows) and 2x3072 x 1024 7.4 against 6.1 (a small matrix).
+    Against the library and the activation kernel from 17 to 64 rows: 2x9728 x 2560 21 to 27
+    against 30 to 34, 2x12288 x 4096 45 to 48 against 48 to 53, 2x17408 x 5120 67 to 86 against
+    78 to 93, 2x25600 x 5120 91 to 105 against 94 to 107, 2x3072 x 1024 9.3 to 12.8 against
+    13.8 to 14.3 (2x6144 x 2048 at 64 rows alone loses, 20.9 against 19.8).  A workgroup of the
+    rows kernel sees its gate rows and, ``n_half`` rows further, its up rows through one
+    descriptor, which spans at most 2 GB."""
     few = rows <= FEW_ROWS
     fits = (n_half + 64) * row_stride * 2 < 2 ** 31
-    if fits and ((not aliased_rows(k) and n_half >= 4096) if few else k <= 4096):
+    if fits and (not few or (not aliased_rows(k) and n_half >= 4096)):
         return Product("rows", 1, 2)
     return Product("skinny") if few else Product("library")

@@ -59,8 +59,11 @@ def test_rows_of_a_power_of_two_length_and_small_matrices_keep_the_other_kernels
     assert plan.plan_projection(8, q + 2 * kv, hidden).kernel == "rows"
     assert plan.plan_projection(8, VOCAB, hidden).kernel == "skinny"
     assert plan.plan_gated(8, 3072, 1024, 1024).kernel == "skinny"      # a small matrix
-    assert plan.plan_gated(64, 25600, 5120, 5120).kernel == "library"   # wider than 4096
-    assert plan.plan_residual(64, 8192, 8192).kernel == "library"       # wide and shallow
+    assert plan.plan_gated(64, 25600, 5120, 5120).kernel == "rows"      # from 17 rows whatever the width
+    assert plan.plan_residual(64, 8192, 8192).kernel == "library"       # wide, and rows of a power-of-two length
+    assert plan.plan_residual(64, 16384, 4096).kernel == "library"
+    assert plan.plan_residual(64, 5120, 8192) == plan.Product("rows", 4, 2)   # not wide
+    assert plan.plan_residual(64, 10240, 10240).kernel == "rows"        # wide, rows of another length
     assert plan.plan_residual(8, 16384, 8192).kernel == "skinny"
 
 

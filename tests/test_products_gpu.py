@@ -26,8 +26,8 @@ product    1, 8, 16 rows             17, 48, 64 rows                        65, 
 8b down    rows CT1 4w 64x4 c64      rows CT2 4w 32x8 c128                  library
 8b head    skinny                    rows CT2 4w 1187x1 c128                library, float32
 32b qkv    rows CT1 4w 256x1 c40     library                                library
-32b out    rows CT2 4w 64x4 c80      library, float32                       library
-32b g/u    rows GLU 4w 512x1 c50     library float32 + silu_gate            library + silu_gate
+32b out    rows CT2 4w 64x4 c80      rows CT2 4w 64x4 c80                   library
+32b g/u    rows GLU 4w 512x1 c50     rows GLU 4w 512x1 c50                  library + silu_gate
 32b down   rows CT2 4w 64x4 c80      rows CT2 4w 64x4 c80                   library
 32b head   rows CT2 4w 1277x1 c119   rows CT2 4w 1187x1 c128                library, float32
 =========  ========================  =====================================  ===================
@@ -67,8 +67,8 @@ EXPECT = {
     ("8b", "down"): ((R, 4, 1, (4, 64, 64)), (R, 8, 2, (4, 32, 128))),
     ("8b", "head"): (("skinny",), (R, 1, 2, (4, 1187, 128))),
     ("32b", "qkv"): ((R, 1, 1, (4, 256, 40)), ("library",)),
-    ("32b", "out"): ((R, 4, 2, (4, 64, 80)), ("library",)),
-    ("32b", "gate_up"): ((R, 1, 2, (4, 512, 50)), ("library",)),
+    ("32b", "out"): ((R, 4, 2, (4, 64, 80)), (R, 4, 2, (4, 64, 80))),
+    ("32b", "gate_up"): ((R, 1, 2, (4, 512, 50)), (R, 1, 2, (4, 512, 50))),
     ("32b", "down"): ((R, 4, 2, (4, 64, 80)), (R, 4, 2, (4, 64, 80))),
     ("32b", "head"): ((R, 1, 2, (4, 1277, 119)), (R, 1, 2, (4, 1187, 128))),
 }
