@@ -95,18 +95,23 @@ def plan_residual(rows: int, n: int, k: int, units: int = UNITS) -> Product:
 def plan_projection(rows: int, n: int, k: int) -> Product:
     """Any other product of ``rows`` <= 64 (q/k/v; the vocabulary head).
 
-    A head (tall matrix): the rows kernel with 128 columns per workgroup (151936 x 2560: 136 us
-    against the skinny kernel's 154 at 8 rows; 172 against the library's 190 at 64 rows, 149
-    against 174 at 24), except up to 16 rows of aliased rows (x 4096: 239 against 237).
+    A head (tall matrix): the rows kernel with 128 columns per workgroup (151936 x 2560: 137 us
+    against the skinny kernel's 154 at 8 rows; 173 against the library's 186 at 64 rows, 150
+    against 173 at 32; x 5120: 264 against 304 and 303 against 313).  With aliased rows (x 4096)
+    64 columns per workgroup do better (220 against 227 us at 1 row, 230 against 235 at 8, 262
+    against 272 at 32, the skinny kernel 237, 234 and, at 16 rows, 258 against 239), and beyond
+    32 rows the library (274 against 286 and 300 at 64 rows).
     A projection up to 16 rows: the rows kernel (6144 x 2560 at 8 rows 9.3 against the skinny
-    kernel's 10.7 us, 10240 x 5120 21 against 31, 6144 x 4096 13.5 against 16).  Beyond 16
-    rows the library: the rows kernel is within 10 % of it either way (6144 x 2560: 14.4
-    against 15.4 us at 48 rows, 17.2 against 15.5 at 64; 7168 x 5120: 24 against 23 and 30
-    against 24; 10240 x 5120: 28 against 32 and 31 against 33), and the rows of x of a
-    workgroup that covers 64 of many columns weigh most here."""
+    kernel's 10.7 us, 10240 x 5120 21 against 31, 6144 x 4096 14.5 against 16).  Beyond 16
+    rows the library: without K cut over workgroups the rows kernel is within 10 % of it either
+    way (6144 x 2560: 12.2 against 11.8 us at 32 rows, 17.8 against 15.5 at 64), and the rows of
+    x of a workgroup that covers 64 of many columns weigh most here; a consumer that adds
+    partial sums gets them (:func:`plan_summed_later`)."""
     few = rows <= FEW_ROWS
     if n >= TALL:
-        return Product("skinny") if few and aliased_rows(k) else Product("rows", 1, 2)
+        if aliased_rows(k):
+            return Product("rows", 1, 1) if rows <= 32 else Product("library")
+        return Product("rows", 1, 2)
     return Product("rows") if few else Product("library")
 
 

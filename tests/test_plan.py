@@ -57,7 +57,9 @@ def test_rows_of_a_power_of_two_length_and_small_matrices_keep_the_other_kernels
     assert plan.plan_gated(64, inter, hidden, hidden).kernel == "rows"
     assert plan.plan_projection(48, q + 2 * kv, hidden).kernel == "library"
     assert plan.plan_projection(8, q + 2 * kv, hidden).kernel == "rows"
-    assert plan.plan_projection(8, VOCAB, hidden).kernel == "skinny"
+    assert plan.plan_projection(8, VOCAB, hidden) == plan.Product("rows", 1, 1)   # 64 columns a workgroup
+    assert plan.plan_projection(32, VOCAB, hidden) == plan.Product("rows", 1, 1)
+    assert plan.plan_projection(33, VOCAB, hidden).kernel == "library"
     assert plan.plan_gated(8, 3072, 1024, 1024).kernel == "skinny"      # a small matrix
     assert plan.plan_gated(64, 25600, 5120, 5120).kernel == "rows"      # from 17 rows whatever the width
     assert plan.plan_residual(64, 8192, 8192).kernel == "library"       # wide, and rows of a power-of-two length

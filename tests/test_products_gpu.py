@@ -24,7 +24,8 @@ product    1, 8, 16 rows             17, 48, 64 rows                        65, 
 8b out     rows CT1 4w 64x4 c64      rows CT1 4w 64x4 c64                   library
 8b gate/up skinny GLU                rows GLU 4w 256x1 c48                  library + silu_gate
 8b down    rows CT1 4w 64x4 c64      rows CT2 4w 32x8 c128                  library
-8b head    skinny                    rows CT2 4w 1187x1 c128                library, float32
+8b head    rows CT1 4w 2533x1 c60    rows CT1 4w 2374x1 c64 at 17 rows,     library, float32
+                                     library float32 at 48 and 64
 32b qkv    rows CT1 4w 256x1 c40     library                                library
 32b out    rows CT2 4w 64x4 c80      rows CT2 4w 64x4 c80                   library
 32b g/u    rows GLU 4w 512x1 c50     rows GLU 4w 512x1 c50                  library + silu_gate
@@ -65,7 +66,7 @@ EXPECT = {
     ("8b", "out"): ((R, 4, 1, (4, 64, 64)), (R, 4, 1, (4, 64, 64))),
     ("8b", "gate_up"): (("skinny",), (R, 1, 2, (4, 256, 48))),
     ("8b", "down"): ((R, 4, 1, (4, 64, 64)), (R, 8, 2, (4, 32, 128))),
-    ("8b", "head"): (("skinny",), (R, 1, 2, (4, 1187, 128))),
+    ("8b", "head"): ((R, 1, 1, (4, 2533, 60)), {17: (R, 1, 1, (4, 2374, 64)), 48: ("library",), 64: ("library",)}),
     ("32b", "qkv"): ((R, 1, 1, (4, 256, 40)), ("library",)),
     ("32b", "out"): ((R, 4, 2, (4, 64, 80)), (R, 4, 2, (4, 64, 80))),
     ("32b", "gate_up"): ((R, 1, 2, (4, 512, 50)), (R, 1, 2, (4, 512, 50))),
