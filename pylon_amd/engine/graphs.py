@@ -11,7 +11,8 @@ is seen, and a batch is never padded to a larger captured size.
 The launches recorded in a graph must not depend on the requests' lengths: the block
 table has a fixed width, and what a mixer launches may depend on the batch size and on a
 bound on the lengths only (the decode attention kernel shares a request's keys between
-workgroups and waves by it).  That bound is a power of two of at least 1024 tokens.  A
+workgroups and waves by it).  That bound is a power of two of at least 512 tokens (up to
+there one workgroup per token and head is fastest; beyond, the keys are cut).  A
 mixer says through ``decode_signature(rows, bound)`` what of its launches depends on the
 bound; bounds with equal signatures share one graph, and a mixer that does not say is taken
 to depend on the bound itself.  There is one graph per (batch size, signature).
@@ -27,6 +28,8 @@ import torch
 from .batch import StepEntry, build_step, plan_layout
 
 logger = logging.getLogger("pylon")
+
+MIN_BOUND = 512  # the smallest bound on the requests' lengths a graph is captured for
 
 
 class DecodeGraphs:
@@ -60,18 +63,18 @@ class DecodeGraphs:
         return rows, (("bound", bound) if describe is None else describe(rows, bound))
 
     def _bound(self, entries: Seq[StepEntry]) -> int:
-        """The power of two (from 1024) that holds the longest request after this step."""
+        """The power of two (from MIN_BOUND) that holds the longest request after this step."""
         need = max(e.seq.length for e in entries) + 1
-        bound = 1024
+        bound = MIN_BOUND
         while bound < need:
             bound *= 2
         return bound
 
     def bounds(self) -> Tuple[int, ...]:
-        """Every bound a graph may be captured for: the powers of two from 1024 up to the one
-        that holds the longest request the block table has room for."""
+        """Every bound a graph may be captured for: the powers of two from MIN_BOUND up to the
+        one that holds the longest request the block table has room for."""
         longest = self.width * self.manager.page_size
-        out = [1024]
+        out = [MIN_BOUND]
         while out[-1] < longest:
             out.append(out[-1] * 2)
         return tuple(out)

@@ -300,7 +300,7 @@ def test_a_replay_that_raises_leaves_the_cache_as_it_was():
     graphs.chosen, graphs.width, graphs.max_batch = None, 4, 4
     graphs.failed, graphs.replays, graphs.last_logit_slots = set(), 0, None
     block = torch.empty(256, dtype=torch.int32)
-    graphs.captured = {graphs.key(1, 1024): (BrokenGraph(), block, None, None)}
+    graphs.captured = {graphs.key(1, 512): (BrokenGraph(), block, None, None)}
     with pytest.raises(RuntimeError, match="replay failed"):
         graphs.run([StepEntry(a, [7], [0])])
     assert m.free_pages == free and a._pending is None and a.length == 4

@@ -164,12 +164,13 @@ def test_graphs_captured_at_start_up(tmp_path):
     # those of every bound are, by short requests, and a long request then only replays
     big = Runner.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=140, max_requests=3)
     big.enable_graphs(2)
-    assert big.graphs.bounds() == (1024, 2048, 4096)
+    assert big.graphs.bounds() == (512, 1024, 2048, 4096)
     big.capture_graphs(max_tokens=1000)
-    assert set(big.graphs.captured) == {big.graphs.key(1, 1024), big.graphs.key(2, 1024)}
+    assert set(big.graphs.captured) == {big.graphs.key(rows, bound) for rows in (1, 2) for bound in (512, 1024)}
     big.capture_graphs()
-    assert set(big.graphs.captured) == {big.graphs.key(rows, bound) for rows in (1, 2) for bound in (1024, 2048, 4096)}
-    assert len(big.graphs.captured) == 6  # two key/value heads: every bound cuts the keys otherwise
+    assert set(big.graphs.captured) == {big.graphs.key(rows, bound) for rows in (1, 2)
+                                        for bound in (512, 1024, 2048, 4096)}
+    assert len(big.graphs.captured) == 8  # two key/value heads: every bound cuts the keys otherwise
     plain_runner = Runner.from_folder(folder, dtype="bfloat16", page_size=16, num_pages=140, max_requests=3)
     long_prompt = random_tokens(cfg["vocab_size"], 1100, 5)
     outs = []
@@ -177,5 +178,5 @@ def test_graphs_captured_at_start_up(tmp_path):
         seq = r.open("long")
         r.step([StepEntry(seq, long_prompt, [])])
         outs.append(np.concatenate([r.step([StepEntry(seq, [11 + t], [0])]).cpu().numpy() for t in range(4)]))
-    assert len(big.graphs.captured) == 6 and big.graphs.replays >= 6 + 4
+    assert len(big.graphs.captured) == 8 and big.graphs.replays >= 8 + 4
     assert rows_within(outs[0], outs[1], 1e-2)[0]

@@ -78,7 +78,7 @@ LONG = dict(CONFIGS["D"], max_position_embeddings=262144, num_hidden_layers=3, v
 
 def test_start_up_with_graphs_at_a_position_limit_of_262144(gpu, tmp_path):
     """Every decode graph is captured at start-up, in bounded time and memory: bounds on the
-    requests' lengths at which the recorded launches are the same share a graph, so nine bounds
+    requests' lengths at which the recorded launches are the same share a graph, so ten bounds
     make a few graphs per small batch size and two per large one; no graph is captured while
     serving, however long the request."""
     from pylon_amd.engine.engine import Engine
@@ -95,11 +95,11 @@ def test_start_up_with_graphs_at_a_position_limit_of_262144(gpu, tmp_path):
     try:
         runner = engine.runner
         graphs = runner.graphs
-        assert len(graphs.bounds()) == 9 and graphs.bounds()[-1] == 262144
+        assert len(graphs.bounds()) == 10 and graphs.bounds()[0] == 512 and graphs.bounds()[-1] == 262144
         expected = {(rows, (("attention", *ops.decode_launch(rows, cfg["num_key_value_heads"], bound)),))
                     for rows in range(1, 33) for bound in graphs.bounds()}
         assert set(graphs.captured) == expected
-        assert 32 < len(expected) < 32 * 4  # far fewer than one per batch size and bound (288)
+        assert 32 < len(expected) < 32 * 4  # far fewer than one per batch size and bound (320)
         assert runner.manager.num_pages == 32 * (262144 // 256)
         pool = runner.manager.num_pages * 256 * runner.manager.bytes_per_token
         extra = torch.cuda.memory_reserved() - before - pool
@@ -134,12 +134,12 @@ def test_start_up_captures_graphs_up_to_a_configured_length(gpu, tmp_path):
                                 num_pages=64)
     try:
         graphs = engine.runner.graphs
-        assert set(graphs.captured) == {graphs.key(rows, 1024) for rows in range(1, 5)}
+        assert set(graphs.captured) == {graphs.key(rows, bound) for rows in range(1, 5) for bound in (512, 1024)}
         seq = engine.runner.open("long")
         engine.runner.step([StepEntry(seq, random_tokens(cfg["vocab_size"], 2100, 9), [])])
         engine.runner.step([StepEntry(seq, [5], [0])])
         engine.runner.close(seq)
-        assert graphs.key(1, 4096) in graphs.captured and len(graphs.captured) == 5
+        assert graphs.key(1, 4096) in graphs.captured and len(graphs.captured) == 9
     finally:
         engine.close()
 
