@@ -407,7 +407,7 @@ __global__ __launch_bounds__(PYLON_WAVE) void attention_decode_merge_kernel(
   for (int i = 0; i < EPL; ++i) orow[i] = float_to_bf16_bits(o[i] * inv);
 }
 
-static size_t decode_lds_bytes(int n_waves, int gp, int head_dim, bool prep) {
+static inline size_t decode_lds_bytes(int n_waves, int gp, int head_dim, bool prep) {
   return sizeof(float) * decode_lds_floats(n_waves, gp, head_dim) +
          (prep ? sizeof(uint16_t) * static_cast<size_t>(gp) * head_dim + sizeof(float) * n_waves * head_dim +
                      sizeof(uint16_t) * 2 * head_dim
