@@ -15,7 +15,7 @@ the read of the chosen ids by the host; as in serving, a tick queues its step be
 the ids of the step before (they are fed back on the device).  ``value`` is decoded tokens per
 second at the default batch of 8.  The same line carries the prefill of 2,048 tokens (one
 request from its arrival to its first token), the decode step's share of the HBM roofline, and
-under ``points`` decode rates at batch 1 and 64, at contexts of 4,096 and 8,000 tokens, a prompt
+under ``points`` decode rates at batch 1 and 64, at contexts of 2,000, 4,096 and 8,000 tokens, a prompt
 of 8,191 tokens in four portions, a step of 64 decoded tokens beside a 2,048-token portion, and
 two rates over whole requests (queueing, admission and prefill included): ``engine_b8`` with the
 same 128-token prompts and 512 new tokens, ``engine_prefill_heavy_b8`` with 2,048-token prompts
@@ -397,6 +397,7 @@ def main() -> int:
         put("decode_b64", decode_point(runner, cfg, args, 64, prompt_len, few, seed=67))
         if headline:
             # longer contexts: the decode attention's share grows, its keys are cut over workgroups
+            put("decode_b8_ctx2000", decode_point(runner, cfg, args, 8, 2000, 48, seed=15))
             put("decode_b8_ctx4096", decode_point(runner, cfg, args, 8, 4096, 64, seed=11))
             put("decode_b1_ctx8000", decode_point(runner, cfg, args, 1, 8000, 64, seed=12))
             point = decode_point(runner, cfg, args, 64, 4096, 64, seed=13, mixed=True)
