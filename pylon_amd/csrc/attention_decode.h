@@ -380,26 +380,51 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
 
 #undef AD_LOAD
 
-// One wave per (token, query head) merges the partial results of the cuts, in their order.
+// One wave per (token, query head) merges the partial results of the cuts (at most 64), in
+// their order.  Lane c takes the maximum and the sum of cut c, so that all of them come in one
+// trip to memory, and the weighted values come eight cuts a batch, every load of a batch issued
+// before its first addition: the time no longer grows by a trip to memory per cut (32 cuts:
+// 19 us before).
 template <int EPL>
 __global__ __launch_bounds__(PYLON_WAVE) void attention_decode_merge_kernel(
     uint16_t* __restrict__ out, const float* __restrict__ partial, int n_heads, int n_cuts) {
   constexpr int HD = EPL * 64;
+  constexpr int BATCH = 8;
   const int lane = threadIdx.x;
   const size_t row = static_cast<size_t>(blockIdx.y) * n_heads + blockIdx.x;
   const float* prow = partial + row * n_cuts * (HD + 2);
-  float m = -INFINITY;
-  for (int c = 0; c < n_cuts; ++c) m = fmaxf(m, prow[c * (HD + 2) + HD]);
+  float mc = -INFINITY, lc = 0.f;
+  if (lane < n_cuts) {
+    mc = prow[lane * (HD + 2) + HD];
+    lc = prow[lane * (HD + 2) + HD + 1];
+  }
+  float m = mc;
+#pragma unroll
+  for (int off = PYLON_WAVE / 2; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, PYLON_WAVE));
+  const float fc = (lc == 0.f) ? 0.f : expf(mc - m);  // a cut without keys
+  const float wc = lc * fc;
   float l = 0.f, o[EPL];
 #pragma unroll
   for (int i = 0; i < EPL; ++i) o[i] = 0.f;
-  for (int c = 0; c < n_cuts; ++c) {
-    const float* pc = prow + c * (HD + 2);
-    const float lc = pc[HD + 1];
-    const float f = (lc == 0.f) ? 0.f : expf(pc[HD] - m);  // a cut without keys
-    l += lc * f;
+  for (int c0 = 0; c0 < n_cuts; c0 += BATCH) {
+    float v[BATCH][EPL];
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) o[i] = fmaf(pc[lane * EPL + i], f, o[i]);
+    for (int u = 0; u < BATCH; ++u) {
+      const int c = (c0 + u < n_cuts) ? c0 + u : n_cuts - 1;  // past the end: a cut again, unused
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) v[u][i] = prow[c * (HD + 2) + lane * EPL + i];
+    }
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      const int c = c0 + u;
+      const float f = __shfl(fc, c & (PYLON_WAVE - 1), PYLON_WAVE);
+      const float w = __shfl(wc, c & (PYLON_WAVE - 1), PYLON_WAVE);
+      if (c < n_cuts) {
+        l += w;
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) o[i] = fmaf(v[u][i], f, o[i]);
+      }
+    }
   }
   const float inv = 1.0f / l;
   uint16_t* orow = out + row * HD + lane * EPL;

@@ -259,18 +259,18 @@ def _like(q: torch.Tensor, out: Optional[torch.Tensor], name: str) -> torch.Tens
 def decode_cuts(tokens: int, n_kv_heads: int, max_len: Optional[int], units: int = plan.UNITS) -> int:
     """Workgroups that share the keys of one (token, key/value head) before the waves of
     each share theirs: more than one when a few requests would otherwise occupy a fraction of
-    the chip, each with at least 384 keys of ``max_len`` (which may be an upper bound above the
-    true lengths), up to one workgroup per compute unit.  Measured on 256 units with 8
-    key/value heads of 128, one launch with its merge against one workgroup per (token,
-    head): 1 token of 1,000 keys 16.8 us (2 cuts) against 20.7, of 2,000 keys 17.9 (4) against
-    31, of 8,000 keys 28.4 (16) against 44 with 4 cuts; 8 tokens of 1,000 keys 19.8 (2) against
-    24.7, of 2,000 keys 24.7 (4) against 42; 16 tokens of 2,000 keys 35 (2) against 48.  At 500
-    keys one workgroup is as fast (13.3 to 14.3 us); and once the workgroups fill the units
+    the chip.  From 768 keys of ``max_len`` on (which may be an upper bound above the true
+    lengths), each cut at least 192 keys, up to one workgroup per compute unit.  Measured on 256
+    units with 8 key/value heads of 128, the launch with its merge against one workgroup per
+    (token, head): 1 token of 1,000 keys 14.1 us (4 cuts) against 20.6, of 2,000 keys 14.1 (8)
+    against 31, of 8,000 keys 19.1 (32) against 125; 8 tokens of 700 keys 15.2 (4) against 19.7,
+    of 2,000 keys 23.6 (4) against 42; 16 tokens of 2,000 keys 35 (2) against 49.  At 500 keys one
+    workgroup is within a microsecond (13.2 to 14.3 us); and once the workgroups fill the units
     (32 tokens) a cut only adds the second kernel."""
-    if max_len is None:
+    if max_len is None or max_len < 768:
         return 1
     cuts = 1
-    while cuts < 64 and tokens * n_kv_heads * cuts * 2 <= units and cuts * 2 * 384 <= max_len:
+    while cuts < 64 and tokens * n_kv_heads * cuts * 2 <= units and cuts * 2 * 192 <= max_len:
         cuts *= 2
     return cuts
 

@@ -102,15 +102,15 @@ def test_a_projection_whose_consumer_adds_partial_sums_is_cut_over_k_from_17_row
 
 def test_decode_attention_cuts_the_keys_of_few_long_requests_over_workgroups():
     """`ops.decode_cuts` is a pure function of the shape: up to 512 keys one workgroup per
-    (token, head); beyond, powers of two of cuts of at least 384 keys while the workgroups stay
+    (token, head), as up to 767; beyond, powers of two of cuts of at least 192 keys while the workgroups stay
     within the compute units; none once the workgroups fill them."""
     from pylon_amd.kernels import ops
 
     for tokens in (1, 2, 8, 16, 64):
         for bound in (1, 64, 511, 512, 767):
             assert ops.decode_cuts(tokens, 8, bound, 256) == 1
-    assert [ops.decode_cuts(1, 8, b, 256) for b in (768, 1024, 2048, 4096, 8192, 32768, 262144)] == [2, 2, 4, 8, 16, 32, 32]
-    assert [ops.decode_cuts(8, 8, b, 256) for b in (1024, 2048, 4096, 262144)] == [2, 4, 4, 4]
+    assert [ops.decode_cuts(1, 8, b, 256) for b in (768, 1024, 2048, 4096, 8192, 32768, 262144)] == [4, 4, 8, 16, 32, 32, 32]
+    assert [ops.decode_cuts(8, 8, b, 256) for b in (1024, 2048, 4096, 262144)] == [4, 4, 4, 4]
     assert [ops.decode_cuts(16, 8, b, 256) for b in (1024, 8192)] == [2, 2]
     assert ops.decode_cuts(17, 8, 8192, 256) == 1 and ops.decode_cuts(64, 8, 8192, 256) == 1
     assert ops.decode_cuts(8, 8, None, 256) == 1
@@ -120,4 +120,4 @@ def test_decode_attention_cuts_the_keys_of_few_long_requests_over_workgroups():
                 for units in (64, 256, 304):
                     cuts = ops.decode_cuts(tokens, heads, bound, units)
                     assert cuts & (cuts - 1) == 0 and 1 <= cuts <= 64
-                    assert cuts == 1 or (tokens * heads * cuts <= units and cuts * 384 <= bound)
+                    assert cuts == 1 or (tokens * heads * cuts <= units and cuts * 192 <= bound)
