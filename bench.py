@@ -15,7 +15,8 @@ the read of the chosen ids by the host; as in serving, a tick queues its step be
 the ids of the step before (they are fed back on the device).  ``value`` is decoded tokens per
 second at the default batch of 8.  The same line carries the prefill of 2,048 tokens (one
 request from its arrival to its first token), the decode step's share of the HBM roofline, and
-under ``points`` decode rates at batch 1 and 64, at contexts of 2,000, 4,096 and 8,000 tokens, a prompt
+under ``points`` decode rates at batch 1 and 64, with the reference's default sampling options
+instead of greedy, at contexts of 2,000, 4,096 and 8,000 tokens, a prompt
 of 8,191 tokens in four portions, a step of 64 decoded tokens beside a 2,048-token portion, and
 two rates over whole requests (queueing, admission and prefill included): ``engine_b8`` with the
 same 128-token prompts and 512 new tokens, ``engine_prefill_heavy_b8`` with 2,048-token prompts
@@ -109,7 +110,8 @@ class Serving:
     """``batch`` requests of ``prompt_len`` random ids each, brought through the engine to the
     point where every one of them decodes; then ticks can be timed."""
 
-    def __init__(self, runner, cfg, args, batch: int, prompt_len: int, ticks: int, seed: int, room: int = 0):
+    def __init__(self, runner, cfg, args, batch: int, prompt_len: int, ticks: int, seed: int, room: int = 0,
+                 temperature: float = 0.0, top_p: float = 1.0):
         import numpy as np
 
         from pylon_amd.engine.engine import Engine
@@ -126,7 +128,7 @@ class Serving:
         self.ticks = self.new_tokens - prefill_ticks - 8
         if self.ticks < 1:
             raise SystemExit(f"bench.py: {prompt_len}-token prompts leave no room for decode steps")
-        sampling = Sampling(max_new_tokens=self.new_tokens, temperature=0.0)
+        sampling = Sampling(max_new_tokens=self.new_tokens, temperature=temperature, top_p=top_p, seed=seed)
         self.futures = [self.engine.enqueue(self.rng.integers(0, cfg.vocab_size, prompt_len).tolist(), None, sampling)
                         for _ in range(batch)]
         while True:
@@ -190,10 +192,12 @@ class Serving:
         self.engine.close()
 
 
-def decode_point(runner, cfg, args, batch: int, prompt_len: int, steps: int, seed: int, mixed: bool = False) -> dict:
-    """Tokens per second and roofline share of decode steps of ``batch`` requests at this context."""
+def decode_point(runner, cfg, args, batch: int, prompt_len: int, steps: int, seed: int, mixed: bool = False,
+                 temperature: float = 0.0, top_p: float = 1.0) -> dict:
+    """Tokens per second and roofline share of decode steps of ``batch`` requests at this context
+    (greedy, or sampled with a temperature and top-p)."""
     serving = Serving(runner, cfg, args, batch, prompt_len, steps + args.warmup + (24 if mixed else 0), seed,
-                      room=1 if mixed else 0)
+                      room=1 if mixed else 0, temperature=temperature, top_p=top_p)
     elapsed, context = serving.timed_ticks(steps, args.warmup)
     out = {"tokens_per_s": batch * steps / elapsed, "ms": 1e3 * elapsed / steps,
            "bytes": weight_bytes(runner) + context * runner.manager.bytes_per_token, "context": context / batch}
@@ -395,6 +399,10 @@ def main() -> int:
 
         put("decode_b1", decode_point(runner, cfg, args, 1, prompt_len, few, seed=4))
         put("decode_b64", decode_point(runner, cfg, args, 64, prompt_len, few, seed=67))
+        # the reference's default sampling options (/root/reference/src/pylon/api/types.py:6-9)
+        # instead of greedy: one workgroup per row norms, cuts at top-p and draws
+        put("decode_b8_sampled", decode_point(runner, cfg, args, 8, prompt_len, few, seed=68, temperature=0.2,
+                                              top_p=0.95))
         if headline:
             # longer contexts: the decode attention's share grows, its keys are cut over workgroups
             put("decode_b8_ctx2000", decode_point(runner, cfg, args, 8, 2000, 48, seed=15))

@@ -67,14 +67,27 @@ __device__ __forceinline__ void for_each(const float* __restrict__ row, int begi
   if (static_cast<int>(threadIdx.x) < head) f(p[threadIdx.x], begin + static_cast<int>(threadIdx.x));
   const float4* v = reinterpret_cast<const float4*>(p + head);
   const int nv = (n - head) >> 2;
-#pragma unroll 4
-  for (int i = threadIdx.x; i < nv; i += blockDim.x) {
-    const float4 q = v[i];
-    const int base = begin + head + 4 * i;
-    f(q.x, base);
-    f(q.y, base + 1);
-    f(q.z, base + 2);
-    f(q.w, base + 3);
+  // Eight loads of a thread are issued before the first of them is used: a workgroup alone on
+  // its compute unit is bound by what it has in flight.
+  constexpr int DEPTH = 8;
+  for (int i0 = threadIdx.x; i0 < nv; i0 += DEPTH * blockDim.x) {
+    float4 q[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int i = i0 + d * blockDim.x;
+      q[d] = v[i < nv ? i : i0];
+    }
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int i = i0 + d * blockDim.x;
+      if (i < nv) {
+        const int base = begin + head + 4 * i;
+        f(q[d].x, base);
+        f(q[d].y, base + 1);
+        f(q[d].z, base + 2);
+        f(q[d].w, base + 3);
+      }
+    }
   }
   const int tail = head + 4 * nv;
   if (static_cast<int>(threadIdx.x) < n - tail)
