@@ -60,12 +60,16 @@ __device__ __forceinline__ void gr_wait_loads() {
   __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
 }
 
-// Stages of LDS for MT tiles of x and WAVES * CT tiles of w per chunk: as many as fit, at most 4.
+// Stages of LDS for MT tiles of x and WAVES * CT tiles of w per chunk.
 template <int MT, int CT, int WAVES>
 struct GrShape {
   static constexpr int TILES = MT + WAVES * CT;
   static constexpr int STAGE_BYTES = TILES * GR_TILE_BYTES;
-  static constexpr int STAGES = (4 * STAGE_BYTES <= 144 * 1024) ? 4 : 3;
+  // Four stages where they fit and a wave brings one tile of w per chunk; with two tiles a wave
+  // (36 KB a stage and more) three do better by 1 to 2 % (gate/up 2 x 9728 x 2560 at 8 rows:
+  // 19.6 against 20.0 us; the head 139.1 against 140.2), and with one tile a wave three lose
+  // 4 to 7 %; six stages are slower everywhere.
+  static constexpr int STAGES = (4 * STAGE_BYTES <= 144 * 1024 && CT == 1) ? 4 : 3;
 };
 
 // MT: tiles of 16 rows of x (1..4); CT: tiles of 16 rows of w per wave (1 or 2).
