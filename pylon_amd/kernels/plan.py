@@ -117,13 +117,25 @@ def plan_projection(rows: int, n: int, k: int) -> Product:
 
 def plan_summed_later(rows: int, n: int, k: int, units: int = UNITS) -> Product:
     """A projection whose consumer can add float partial sums itself (q/k/v in front of the
-    decode attention that prepares its own operands).  Beyond 16 rows the rows kernel with K
-    cut over workgroups then beats the library, which does not cut K: 6144 x 2560 at 17, 32,
-    48 and 64 rows 9.0, 9.5, 10.8 and 11.7 us (four parts of 128 columns) against 11.0, 11.8,
-    15.3 and 15.5; 6144 x 4096 11.8 to 14.9 against 14.5 to 17.9; 10240 x 5120 (two parts)
-    21.5 to 28.1 against 24.4 to 32.8.  Without a cut, and up to 16 rows, as
-    :func:`plan_projection`."""
-    if FEW_ROWS < rows <= STREAM_ROWS and n < TALL:
+    decode attention that prepares its own operands): K is cut over workgroups where the uncut
+    launch would leave compute units without one.
+
+    Up to 16 rows: workgroups of 64 columns and 2 or 4 parts, as many as keep the workgroups
+    within the units.  At 8 rows 6144 x 2560 takes 7.8 us (2 parts) against 10.3 uncut, 4096 x
+    2048 5.5 (4) against 8.5, 6144 x 4096 12.3 (2) against 14.5, 7168 x 5120 15.0 (2) against
+    17.6; 10240 x 5120 stays uncut (19.8 against 20.1).  With what the attention kernel then
+    pays for adding them, a whole step at the Qwen3-4B shape, batch 8: 2.603 -> 2.531 ms.
+    From 17 to 64 rows the rows kernel so cut beats the library, which does not cut K: 6144 x
+    2560 at 17, 32, 48 and 64 rows 9.0, 9.5, 10.8 and 11.7 us (four parts of 128 columns) against
+    11.0, 11.8, 15.3 and 15.5; 6144 x 4096 11.8 to 14.9 against 14.5 to 17.9; 10240 x 5120 (two
+    parts) 21.5 to 28.1 against 24.4 to 32.8.  Without a cut as :func:`plan_projection`."""
+    if n < TALL and rows <= FEW_ROWS:
+        groups, parts = -(-n // 64), 1
+        while parts < 4 and 2 * parts * groups <= units and k // (2 * parts) >= 256:
+            parts *= 2
+        if parts > 1:
+            return Product("rows", parts, 1)
+    elif n < TALL and rows <= STREAM_ROWS:
         parts, col_tiles = rows_split(n, k, rows, units)
         if parts > 1:
             return Product("rows", parts, col_tiles)

@@ -83,21 +83,28 @@ def test_parts_are_powers_of_two_and_independent_of_the_row_count_within_a_class
             assert parts & (parts - 1) == 0 and col_tiles in (1, 2)
 
 
-def test_a_projection_whose_consumer_adds_partial_sums_is_cut_over_k_from_17_rows():
-    """q/k/v in front of the decode attention that prepares its own operands: up to 16 rows and
-    for a matrix that is not cut as `plan_projection`; from 17 to 64 rows the rows kernel with
-    K cut (4B and 8B: four parts of 128 columns; 32B: two)."""
-    for name, want in (("4b", (4, 2)), ("8b", (4, 2)), ("32b", (2, 2))):
+def test_a_projection_whose_consumer_adds_partial_sums_is_cut_over_k():
+    """q/k/v in front of the decode attention that prepares its own operands: up to 16 rows two
+    or four parts of 64 columns where that keeps the workgroups within the compute units (4B,
+    8B: two; 32B: none); from 17 to 64 rows the split of a residual product (4B and 8B: four
+    parts of 128 columns; 32B: two); a matrix that is not cut goes as `plan_projection` says."""
+    for name, few, many in (("4b", (2, 1), (4, 2)), ("8b", (2, 1), (4, 2)), ("32b", None, (2, 2)),
+                            ("1.7b", (4, 1), (4, 1))):
         hidden, q, kv, _ = SIZES[name]
         n = q + 2 * kv
         for rows in (1, 8, 16):
-            assert plan.plan_summed_later(rows, n, hidden) == plan.plan_projection(rows, n, hidden)
+            c = plan.plan_summed_later(rows, n, hidden)
+            if few is None:
+                assert c == plan.plan_projection(rows, n, hidden)
+            else:
+                assert (c.kernel, c.parts, c.col_tiles) == ("rows", *few), (name, rows, c)
         for rows in (17, 40, 64):
             c = plan.plan_summed_later(rows, n, hidden)
-            assert (c.kernel, c.parts, c.col_tiles) == ("rows", *want), (name, rows, c)
+            assert (c.kernel, c.parts, c.col_tiles) == ("rows", *many), (name, rows, c)
     # a head is never cut (nothing behind it adds), nor is a matrix with too little K per part
-    assert plan.plan_summed_later(40, VOCAB, 2560) == plan.plan_projection(40, VOCAB, 2560)
-    assert plan.plan_summed_later(40, 6144, 256).parts == 1
+    for rows in (8, 40):
+        assert plan.plan_summed_later(rows, VOCAB, 2560) == plan.plan_projection(rows, VOCAB, 2560)
+        assert plan.plan_summed_later(rows, 6144, 256).parts == 1
 
 
 def test_decode_attention_cuts_the_keys_of_few_long_requests_over_workgroups():
