@@ -12,14 +12,16 @@
 // leave the cumulative sum short of its target.
 //
 // argmax alone runs in two launches, many workgroups per row and then a merge.  sample
-// runs one workgroup per row in about five passes over the row:
-//   1. the maximum (and its index);
-//   2. the total mass and, for top_p < 1, a histogram of mass over 2048 bins that are
-//      monotone in the logit, which names the one bin the top-p boundary falls into;
-//   3. the tokens of that bin are gathered in LDS and the exact boundary key is found
-//      there by bisection (if they do not fit, by bisection with passes over the row);
-//   4. the cumulative mass of kept tokens in index order, narrowed from the row to a
-//      sixteenth of it twice and then scanned.
+// runs one workgroup per row; its sixteen waves each walk one stretch of the row, and what
+// bounds a pass is the arithmetic per element, not the reading:
+//   1. the maximum;
+//   2. the mass of every stretch and, for top_p < 1, a histogram of mass over 2048 bins that
+//      are monotone in the logit, which names the one bin the top-p boundary falls into;
+//   3. the tokens of that bin are gathered in LDS (beside them, per stretch, the mass of the
+//      bins before) and the exact boundary key is found there by bisection (if they do not
+//      fit, by bisection with passes over the row);
+//   4. the cumulative mass of kept tokens in index order: the stretch by the totals that the
+//      earlier passes left, then a sixteenth of it, then a scan.
 #include "common.h"
 #include "no_alloc.h"
 
@@ -244,9 +246,18 @@ __device__ __forceinline__ u64 block_sum_u64(u64 v, u64* scratch) {
   return total;
 }
 
+// floor(f) for 0 <= f <= 2^40, in five instructions: the upper word by a truncating conversion,
+// the rest exactly (f has 24 significant bits), truncated again.
+__device__ __forceinline__ u64 floor_u64(float f) {
+  const uint32_t hi = static_cast<uint32_t>(f * 0x1p-32f);
+  const float rest = fmaf(-static_cast<float>(hi), 0x1p32f, f);
+  return (static_cast<u64>(hi) << 32) | static_cast<uint32_t>(rest);
+}
+
 // A token's probability mass relative to the most likely one, in units of 2^-40.
-__device__ __forceinline__ u64 mass_of(float x, float mx, float inv_temp) {
-  return static_cast<u64>(expf((x - mx) * inv_temp) * FIXED_ONE);
+// `rate` is log2(e) / temperature.
+__device__ __forceinline__ u64 mass_of(float x, float mx, float rate) {
+  return floor_u64(__builtin_amdgcn_exp2f((x - mx) * rate) * FIXED_ONE);
 }
 
 // Bin 0 holds the most likely tokens; a larger logit never lands in a later bin.
@@ -266,13 +277,38 @@ __device__ __forceinline__ float4 load_four(const float* __restrict__ row, int i
   return v;
 }
 
+// f(value, index) for the elements of row[s0, s1) over the lanes of one wave (s0 a multiple of
+// 4), four loads of a lane issued before the first is used.  The last group of four may reach
+// past s1: f then sees -inf at an index >= s1.
+template <typename F>
+__device__ __forceinline__ void wave_each(const float* __restrict__ row, int s0, int s1, bool aligned, F f) {
+  const int lane = threadIdx.x & (PYLON_WAVE - 1);
+  constexpr int DEPTH = 4, STEP = 4 * PYLON_WAVE;
+  for (int i0 = s0 + 4 * lane; i0 < s1; i0 += DEPTH * STEP) {
+    float4 q[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) q[d] = load_four(row, i0 + d * STEP, s1, aligned);
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int i = i0 + d * STEP;
+      f(q[d].x, i);
+      f(q[d].y, i + 1);
+      f(q[d].z, i + 2);
+      f(q[d].w, i + 3);
+    }
+  }
+}
+
+// The row is walked in sixteen consecutive stretches, one per wave, the same stretches by which
+// pass 4 narrows first: what a wave sums over its stretch in an earlier pass is that level's total.
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     int* __restrict__ out, const float* __restrict__ logits, int vocab, long long row_stride,
     const float* __restrict__ temperature, const float* __restrict__ top_p,
     const float* __restrict__ uniform, int* __restrict__ chosen, const int* __restrict__ place) {
-  // The histogram first; once the boundary bin is known, that bin's tokens (key, mass).
-  __shared__ __align__(16) unsigned char pool[CANDIDATES * (sizeof(uint32_t) + sizeof(u64))];
-  __shared__ ArgBest best_scratch[SAMPLE_WAVES];
+  // The histogram first; once the boundary bin is known, that bin's tokens (key, index, mass).
+  __shared__ __align__(16) unsigned char pool[CANDIDATES * (2 * sizeof(uint32_t) + sizeof(u64))];
+  __shared__ float max_scratch[SAMPLE_WAVES];
+  __shared__ int index_scratch[SAMPLE_WAVES];
   __shared__ u64 sum_scratch[SAMPLE_WAVES];
   __shared__ u64 seg_total[SAMPLE_WAVES];
   __shared__ u64 shared_mass[2];  // [0]: mass in the bins before the boundary bin; [1]: kept mass
@@ -284,21 +320,48 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const int r = blockIdx.x;
   const float* row = logits + static_cast<size_t>(r) * row_stride;
   const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
+  const bool aligned = (reinterpret_cast<uintptr_t>(row) & 15) == 0;
   const float temp = temperature[r];
+  int first_seg = (vocab + SAMPLE_WAVES - 1) / SAMPLE_WAVES;
+  first_seg = (first_seg + 4 * PYLON_WAVE - 1) / (4 * PYLON_WAVE) * (4 * PYLON_WAVE);
+  const int w0 = wave * first_seg < vocab ? wave * first_seg : vocab;  // this wave's stretch
+  const int w1 = w0 + first_seg < vocab ? w0 + first_seg : vocab;
 
-  // pass 1
-  const ArgBest top = block_argbest(row, 0, vocab, best_scratch);
-  const int top_index = top.index == 0x7fffffff ? 0 : top.index;
-  const float mx = top.value;
+  // pass 1: the maximum (NaN counts as -inf: the hardware's maximum passes the other operand)
+  float mx = -INFINITY;
+  wave_each(row, w0, w1, aligned, [&](float x, int) { mx = fmaxf(mx, x); });
+  for (int off = PYLON_WAVE / 2; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, PYLON_WAVE));
+  if (lane == 0) max_scratch[wave] = mx;
+  __syncthreads();
+  for (int i = 0; i < SAMPLE_WAVES; ++i) mx = fmaxf(mx, max_scratch[i]);
+  // The lowest index that holds the maximum (0 for an empty row): what a row without a
+  // temperature takes, and what never leaves out[] unset.
+  auto top_index = [&]() -> int {
+    int best = 0x7fffffff;
+    wave_each(row, w0, w1, aligned, [&](float x, int i) {
+      if (clean(x) == mx && i < w1 && i < best) best = i;
+    });
+    for (int off = PYLON_WAVE / 2; off > 0; off >>= 1) {
+      const int other = __shfl_xor(best, off, PYLON_WAVE);
+      best = other < best ? other : best;
+    }
+    __syncthreads();
+    if (lane == 0) index_scratch[wave] = best;
+    __syncthreads();
+    for (int i = 0; i < SAMPLE_WAVES; ++i) best = index_scratch[i] < best ? index_scratch[i] : best;
+    return best == 0x7fffffff ? 0 : best;
+  };
   if (temp <= 0.f || !(mx > -INFINITY) || !(mx < INFINITY)) {
-    if (threadIdx.x == 0) emit(out, chosen, place, r, top_index);
+    const int index = top_index();
+    if (threadIdx.x == 0) emit(out, chosen, place, r, index);
     return;
   }
   const float inv_temp = 1.0f / temp;
+  const float rate = inv_temp * 1.44269504088896340736f;
   const float p = top_p[r];
   const bool restricted = p < 1.0f;
 
-  // pass 2
+  // pass 2: the mass of every stretch and, for top_p < 1, the histogram
   u64* hist = reinterpret_cast<u64*>(pool);
   if (restricted) {
     for (int b = threadIdx.x; b < BINS; b += SAMPLE_THREADS) hist[b] = 0;
@@ -310,16 +373,25 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     __syncthreads();
   }
   u64 zq = 0;
-  for_each(row, 0, vocab, [&](float x, int) {
+  wave_each(row, w0, w1, aligned, [&](float x, int) {
     x = clean(x);
-    const u64 q = mass_of(x, mx, inv_temp);
+    const u64 q = mass_of(x, mx, rate);
     zq += q;
     if (restricted && q != 0) atomicAdd(&hist[bin_of(x, mx, inv_temp)], q);
   });
-  zq = block_sum_u64(zq, sum_scratch);  // >= 2^40: the maximum itself
+  zq = wave_sum_u64(zq);
+  __syncthreads();
+  if (lane == 0) seg_total[wave] = zq;
+  __syncthreads();
+  zq = 0;
+  for (int i = 0; i < SAMPLE_WAVES; ++i) zq += seg_total[i];  // >= 2^40: the maximum itself
 
   uint32_t threshold = 0;  // tokens with key >= threshold are kept
   u64 kept_mass = zq;
+  auto kept_mass_of = [&](float x) -> u64 {
+    x = clean(x);
+    return float_key(x) >= threshold ? mass_of(x, mx, rate) : 0;
+  };
   if (restricted) {
     u64 target = static_cast<u64>(static_cast<double>(p) * static_cast<double>(zq));
     if (target >= zq) target = zq - 1;
@@ -348,13 +420,21 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const u64 before_bin = shared_mass[0];
     __syncthreads();  // the histogram is read; its memory now takes the bin's tokens
 
-    // pass 3
+    // pass 3: the boundary bin's tokens into LDS; beside them what this wave's stretch holds in
+    // the bins before, which is kept whatever the threshold turns out to be
     uint32_t* cand_key = reinterpret_cast<uint32_t*>(pool);
-    u64* cand_mass = reinterpret_cast<u64*>(pool + CANDIDATES * sizeof(uint32_t));
-    for_each(row, 0, vocab, [&](float x, int) {
+    uint32_t* cand_index = reinterpret_cast<uint32_t*>(pool + CANDIDATES * sizeof(uint32_t));
+    u64* cand_mass = reinterpret_cast<u64*>(pool + 2 * CANDIDATES * sizeof(uint32_t));
+    u64 above = 0;
+    wave_each(row, w0, w1, aligned, [&](float x, int i) {
       x = clean(x);
-      if (bin_of(x, mx, inv_temp) != boundary) return;
-      const u64 q = mass_of(x, mx, inv_temp);
+      const int bin = bin_of(x, mx, inv_temp);
+      if (bin > boundary) return;
+      const u64 q = mass_of(x, mx, rate);
+      if (bin < boundary) {
+        above += q;
+        return;
+      }
       if (q == 0) return;
       const uint32_t key = float_key(x);
       atomicMin(&key_range[0], key);
@@ -362,9 +442,11 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       const int at = atomicAdd(&cand_count, 1);
       if (at < CANDIDATES) {
         cand_key[at] = key;
+        cand_index[at] = static_cast<uint32_t>(i);
         cand_mass[at] = q;
       }
     });
+    above = wave_sum_u64(above);
     __syncthreads();
     const int count = cand_count;
     // The smallest key k with (mass of keys > k) <= target lies in [lo, hi]: at hi only the
@@ -374,11 +456,11 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       if (wave == 0) {
         while (lo < hi) {
           const uint32_t mid = lo + (hi - lo) / 2;
-          u64 above = 0;
+          u64 over = 0;
           for (int j = lane; j < count; j += PYLON_WAVE)
-            if (cand_key[j] > mid) above += cand_mass[j];
-          above = before_bin + wave_sum_u64(above);
-          if (above <= target)
+            if (cand_key[j] > mid) over += cand_mass[j];
+          over = before_bin + wave_sum_u64(over);
+          if (over <= target)
             hi = mid;
           else
             lo = mid + 1;
@@ -395,62 +477,67 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       __syncthreads();
       threshold = shared_threshold;
       kept_mass = shared_mass[1];
+      // this stretch's kept mass: the bins before, and the bin's tokens from the threshold up
+      u64 mine = 0;
+      for (int j = lane; j < count; j += PYLON_WAVE) {
+        const int at = static_cast<int>(cand_index[j]);
+        if (cand_key[j] >= threshold && at >= w0 && at < w1) mine += cand_mass[j];
+      }
+      mine = above + wave_sum_u64(mine);
+      if (lane == 0) seg_total[wave] = mine;
     } else {
       // More tokens in one bin than LDS holds (thousands of near-equal logits): bisect
       // with a pass over the row for each probe.
       while (lo < hi) {
         const uint32_t mid = lo + (hi - lo) / 2;
-        u64 above = 0;
-        for_each(row, 0, vocab, [&](float x, int) {
+        u64 over = 0;
+        wave_each(row, w0, w1, aligned, [&](float x, int) {
           x = clean(x);
-          if (float_key(x) > mid) above += mass_of(x, mx, inv_temp);
+          if (float_key(x) > mid) over += mass_of(x, mx, rate);
         });
-        above = block_sum_u64(above, sum_scratch);
-        if (above <= target)
+        over = block_sum_u64(over, sum_scratch);
+        if (over <= target)
           hi = mid;
         else
           lo = mid + 1;
       }
       threshold = lo;
       u64 kept = 0;
-      for_each(row, 0, vocab, [&](float x, int) {
-        x = clean(x);
-        if (float_key(x) >= threshold) kept += mass_of(x, mx, inv_temp);
-      });
-      kept_mass = block_sum_u64(kept, sum_scratch);
+      wave_each(row, w0, w1, aligned, [&](float x, int) { kept += kept_mass_of(x); });
+      kept = wave_sum_u64(kept);
+      __syncthreads();
+      if (lane == 0) seg_total[wave] = kept;
+      __syncthreads();
+      kept_mass = 0;
+      for (int i = 0; i < SAMPLE_WAVES; ++i) kept_mass += seg_total[i];
     }
+    __syncthreads();
   }
 
   // pass 4: the first index, in index order, at which the cumulative kept mass exceeds
-  // u * (kept mass).
+  // u * (kept mass): narrowed to one of sixteen stretches (the first time by the totals the
+  // passes above left), then to a sixteenth of that, then scanned.
   float u = uniform[r];
   u = u < 0.f ? 0.f : u;
   u64 target = static_cast<u64>(static_cast<double>(u) * static_cast<double>(kept_mass));
   if (target >= kept_mass) target = kept_mass - 1;
-  const bool aligned = (reinterpret_cast<uintptr_t>(row) & 15) == 0;
-  auto kept_mass_of = [&](float x) -> u64 {
-    x = clean(x);
-    return float_key(x) >= threshold ? mass_of(x, mx, inv_temp) : 0;
-  };
   int begin = 0, end = vocab;
   u64 before = 0;
-  bool lost = false;
+  bool lost = false, have_totals = true;
   while (end - begin > 4 * PYLON_WAVE * 4) {
-    // sixteen consecutive stretches, one per wave
     int seg = (end - begin + SAMPLE_WAVES - 1) / SAMPLE_WAVES;
     seg = (seg + 4 * PYLON_WAVE - 1) / (4 * PYLON_WAVE) * (4 * PYLON_WAVE);
-    const int s0 = begin + wave * seg;
-    const int s1 = s0 + seg < end ? s0 + seg : end;
-    u64 mine = 0;
-#pragma unroll 4
-    for (int i = s0 + 4 * lane; i < s1; i += 4 * PYLON_WAVE) {
-      const float4 v = load_four(row, i, s1, aligned);
-      mine += kept_mass_of(v.x) + kept_mass_of(v.y) + kept_mass_of(v.z) + kept_mass_of(v.w);
+    if (!have_totals) {
+      const int s0 = begin + wave * seg < end ? begin + wave * seg : end;
+      const int s1 = s0 + seg < end ? s0 + seg : end;
+      u64 mine = 0;
+      wave_each(row, s0, s1, aligned, [&](float x, int) { mine += kept_mass_of(x); });
+      mine = wave_sum_u64(mine);
+      __syncthreads();
+      if (lane == 0) seg_total[wave] = mine;
+      __syncthreads();
     }
-    mine = wave_sum_u64(mine);
-    __syncthreads();
-    if (lane == 0) seg_total[wave] = mine;
-    __syncthreads();
+    have_totals = false;
     int pick = -1;
     for (int w = 0; w < SAMPLE_WAVES; ++w) {
       const u64 t = seg_total[w];
@@ -468,7 +555,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     end = begin + seg < end ? begin + seg : end;
   }
   if (lost) {  // cannot happen while the masses are summed as integers; never leave out[] unset
-    if (threadIdx.x == 0) emit(out, chosen, place, r, top_index);
+    const int index = top_index();
+    if (threadIdx.x == 0) emit(out, chosen, place, r, index);
     return;
   }
   if (wave == 0) {
@@ -499,7 +587,15 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         before += __shfl(scan, PYLON_WAVE - 1, PYLON_WAVE);
       }
     }
-    if (lane == 0) emit(out, chosen, place, r, found < 0 ? top_index : found);
+    if (lane == 0) {
+      shared_bin = found;
+      if (found >= 0) emit(out, chosen, place, r, found);
+    }
+  }
+  __syncthreads();
+  if (shared_bin < 0) {  // cannot happen either; never leave out[] unset
+    const int index = top_index();
+    if (threadIdx.x == 0) emit(out, chosen, place, r, index);
   }
 }
 
