@@ -279,9 +279,12 @@ __device__ __forceinline__ float4 load_four(const float* __restrict__ row, int i
 
 // f(value, index) for the elements of row[s0, s1) over the lanes of one wave (s0 a multiple of
 // 4), four loads of a lane issued before the first is used.  The last group of four may reach
-// past s1: f then sees -inf at an index >= s1.
-template <typename F>
-__device__ __forceinline__ void wave_each(const float* __restrict__ row, int s0, int s1, bool aligned, F f) {
+// past s1: f then sees -inf at an index >= s1.  A wave's 256 consecutive elements are passed
+// over where none of them exceeds `above` (NaN does not): the logits of a trained model lie
+// mostly far below the largest, where a pass has nothing to do.
+template <bool SKIP, typename F>
+__device__ __forceinline__ void wave_each(const float* __restrict__ row, int s0, int s1, bool aligned, float above,
+                                          F f) {
   const int lane = threadIdx.x & (PYLON_WAVE - 1);
   constexpr int DEPTH = 4, STEP = 4 * PYLON_WAVE;
   for (int i0 = s0 + 4 * lane; i0 < s1; i0 += DEPTH * STEP) {
@@ -291,6 +294,7 @@ __device__ __forceinline__ void wave_each(const float* __restrict__ row, int s0,
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       const int i = i0 + d * STEP;
+      if (SKIP && __ballot(fmaxf(fmaxf(q[d].x, q[d].y), fmaxf(q[d].z, q[d].w)) > above) == 0) continue;
       f(q[d].x, i);
       f(q[d].y, i + 1);
       f(q[d].z, i + 2);
@@ -329,7 +333,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 
   // pass 1: the maximum (NaN counts as -inf: the hardware's maximum passes the other operand)
   float mx = -INFINITY;
-  wave_each(row, w0, w1, aligned, [&](float x, int) { mx = fmaxf(mx, x); });
+  wave_each<false>(row, w0, w1, aligned, 0.f, [&](float x, int) { mx = fmaxf(mx, x); });
   for (int off = PYLON_WAVE / 2; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, PYLON_WAVE));
   if (lane == 0) max_scratch[wave] = mx;
   __syncthreads();
@@ -338,7 +342,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   // temperature takes, and what never leaves out[] unset.
   auto top_index = [&]() -> int {
     int best = 0x7fffffff;
-    wave_each(row, w0, w1, aligned, [&](float x, int i) {
+    wave_each<false>(row, w0, w1, aligned, 0.f, [&](float x, int i) {
       if (clean(x) == mx && i < w1 && i < best) best = i;
     });
     for (int off = PYLON_WAVE / 2; off > 0; off >>= 1) {
@@ -372,8 +376,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     }
     __syncthreads();
   }
+  // 2^-41.1 of the largest mass is less than one unit: nothing at or below this logit has mass
+  const float massless = mx - 28.5f * temp;
   u64 zq = 0;
-  wave_each(row, w0, w1, aligned, [&](float x, int) {
+  wave_each<true>(row, w0, w1, aligned, massless, [&](float x, int) {
     x = clean(x);
     const u64 q = mass_of(x, mx, rate);
     zq += q;
@@ -395,24 +401,26 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   if (restricted) {
     u64 target = static_cast<u64>(static_cast<double>(p) * static_cast<double>(zq));
     if (target >= zq) target = zq - 1;
-    // The boundary bin: mass before it <= target < mass before it + its own mass.
-    if (wave == 0) {
-      constexpr int PER_LANE = BINS / PYLON_WAVE;
-      u64 mine = 0;
-      for (int j = 0; j < PER_LANE; ++j) mine += hist[lane * PER_LANE + j];
-      u64 scan = mine;
+    // The boundary bin: mass before it <= target < mass before it + its own mass.  Every
+    // thread takes two neighbouring bins; the waves' sums meet in LDS.
+    {
+      static_assert(BINS == 2 * SAMPLE_THREADS, "two bins a thread");
+      const u64 h0 = hist[2 * threadIdx.x], h1 = hist[2 * threadIdx.x + 1];
+      u64 scan = h0 + h1;
       for (int off = 1; off < PYLON_WAVE; off <<= 1) {
         const u64 up = __shfl_up(scan, off, PYLON_WAVE);
         if (lane >= off) scan += up;
       }
-      u64 before = scan - mine;
-      for (int j = 0; j < PER_LANE; ++j) {
-        const u64 h = hist[lane * PER_LANE + j];
-        if (before <= target && target < before + h) {
-          shared_bin = lane * PER_LANE + j;
-          shared_mass[0] = before;
-        }
-        before += h;
+      if (lane == PYLON_WAVE - 1) sum_scratch[wave] = scan;
+      __syncthreads();
+      u64 before = scan - (h0 + h1);
+      for (int i = 0; i < wave; ++i) before += sum_scratch[i];
+      if (before <= target && target < before + h0) {
+        shared_bin = 2 * threadIdx.x;
+        shared_mass[0] = before;
+      } else if (before + h0 <= target && target < before + h0 + h1) {
+        shared_bin = 2 * threadIdx.x + 1;
+        shared_mass[0] = before + h0;
       }
     }
     __syncthreads();
@@ -425,8 +433,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     uint32_t* cand_key = reinterpret_cast<uint32_t*>(pool);
     uint32_t* cand_index = reinterpret_cast<uint32_t*>(pool + CANDIDATES * sizeof(uint32_t));
     u64* cand_mass = reinterpret_cast<u64*>(pool + 2 * CANDIDATES * sizeof(uint32_t));
+    // logits this far below the largest lie behind the boundary bin, whatever bin_of rounds to
+    const float behind = mx - (static_cast<float>(boundary) + 1.5f) * (BIN_RANGE / BINS) * temp;
     u64 above = 0;
-    wave_each(row, w0, w1, aligned, [&](float x, int i) {
+    wave_each<true>(row, w0, w1, aligned, behind, [&](float x, int i) {
       x = clean(x);
       const int bin = bin_of(x, mx, inv_temp);
       if (bin > boundary) return;
@@ -453,18 +463,27 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     // earlier bins are above, at lo - 1 the whole boundary bin would be as well.
     uint32_t lo = key_range[0], hi = key_range[1];
     if (count <= CANDIDATES) {
+      // Sixteen probes a round, one per wave, spread evenly over [lo, hi): the mass above a
+      // probe falls as the probe rises, so the answer lies between the last probe that has
+      // too much above it and the first that has not.
+      while (lo < hi) {
+        const uint32_t mid =
+            lo + static_cast<uint32_t>(static_cast<u64>(hi - lo) * (wave + 1) / (SAMPLE_WAVES + 1));
+        u64 over = 0;
+        for (int j = lane; j < count; j += PYLON_WAVE)
+          if (cand_key[j] > mid) over += cand_mass[j];
+        over = before_bin + wave_sum_u64(over);
+        __syncthreads();
+        if (lane == 0) index_scratch[wave] = over <= target ? 1 : 0;
+        __syncthreads();
+        int first = 0;
+        while (first < SAMPLE_WAVES && index_scratch[first] == 0) ++first;
+        const uint32_t span = hi - lo;
+        if (first < SAMPLE_WAVES)
+          hi = lo + static_cast<uint32_t>(static_cast<u64>(span) * (first + 1) / (SAMPLE_WAVES + 1));
+        if (first > 0) lo = lo + static_cast<uint32_t>(static_cast<u64>(span) * first / (SAMPLE_WAVES + 1)) + 1;
+      }
       if (wave == 0) {
-        while (lo < hi) {
-          const uint32_t mid = lo + (hi - lo) / 2;
-          u64 over = 0;
-          for (int j = lane; j < count; j += PYLON_WAVE)
-            if (cand_key[j] > mid) over += cand_mass[j];
-          over = before_bin + wave_sum_u64(over);
-          if (over <= target)
-            hi = mid;
-          else
-            lo = mid + 1;
-        }
         u64 kept = 0;
         for (int j = lane; j < count; j += PYLON_WAVE)
           if (cand_key[j] >= lo) kept += cand_mass[j];
@@ -491,7 +510,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       while (lo < hi) {
         const uint32_t mid = lo + (hi - lo) / 2;
         u64 over = 0;
-        wave_each(row, w0, w1, aligned, [&](float x, int) {
+        wave_each<true>(row, w0, w1, aligned, massless, [&](float x, int) {
           x = clean(x);
           if (float_key(x) > mid) over += mass_of(x, mx, rate);
         });
@@ -503,7 +522,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       }
       threshold = lo;
       u64 kept = 0;
-      wave_each(row, w0, w1, aligned, [&](float x, int) { kept += kept_mass_of(x); });
+      wave_each<true>(row, w0, w1, aligned, massless, [&](float x, int) { kept += kept_mass_of(x); });
       kept = wave_sum_u64(kept);
       __syncthreads();
       if (lane == 0) seg_total[wave] = kept;
@@ -531,7 +550,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       const int s0 = begin + wave * seg < end ? begin + wave * seg : end;
       const int s1 = s0 + seg < end ? s0 + seg : end;
       u64 mine = 0;
-      wave_each(row, s0, s1, aligned, [&](float x, int) { mine += kept_mass_of(x); });
+      wave_each<true>(row, s0, s1, aligned, massless, [&](float x, int) { mine += kept_mass_of(x); });
       mine = wave_sum_u64(mine);
       __syncthreads();
       if (lane == 0) seg_total[wave] = mine;

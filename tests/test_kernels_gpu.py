@@ -766,6 +766,35 @@ def test_sampling_with_thousands_of_equal_logits_at_the_boundary(ops):
     _check_draws(ops, logits[1:2].repeat(3, 1), temps, torch.full((3,), 0.7), us, plain)
 
 
+def test_sampling_where_most_of_the_row_has_no_mass(ops):
+    """Logits as a trained model's: a handful of tokens carry all the mass and whole stretches
+    of the row lie too far below to have any, which the passes step over 256 tokens at a time.
+    The draws are still the plain rule's, from the first stretch to the last token."""
+    from tests.plain import qwen3 as plain
+
+    vocab = 70001
+    gen = torch.Generator().manual_seed(11)
+    logits = -40.0 - torch.rand((4, vocab), generator=gen)
+    for r, places in enumerate(([5, 20000, 70000], [0, 1, 2, 3], [4352, 4353, 35000, 69999], [12345])):
+        logits[r, places] = torch.tensor([1.0, 0.5, 0.2, -0.3])[: len(places)]
+    # a stretch with a little mass at temperature 1 and none at 0.2 (no two alike: a tie at the
+    # top-p boundary is kept whole by the kernel and cut by the plain rule)
+    logits[2, 60000:60300] = -6.0 - 2.0 * torch.rand(300, generator=gen)
+    for temp, top_p in ((1.0, 1.0), (1.0, 0.9), (0.2, 0.95), (0.2, 1.0), (2.0, 0.5)):
+        temps, tops = torch.full((4,), temp), torch.full((4,), top_p)
+        for trial in range(6):
+            us = torch.rand(4, generator=torch.Generator().manual_seed(50 + trial))
+            _check_draws(ops, logits, temps, tops, us, plain)
+        # the ends of the kept set
+        first = ops.sample(logits.to(DEV), temps.to(DEV), tops.to(DEV), torch.zeros(4, device=DEV)).cpu().tolist()
+        last = ops.sample(logits.to(DEV), temps.to(DEV), tops.to(DEV),
+                          torch.full((4,), 1.0 - 2 ** -24).to(DEV)).cpu().tolist()
+        for r in range(4):
+            p = plain.sampling_distribution(f64(logits)[r], temp, top_p)
+            kept = np.nonzero(p > 2.0 ** -40)[0]
+            assert first[r] == int(kept[0]) and last[r] == int(kept[-1]), (temp, top_p, r, first[r], last[r])
+
+
 @pytest.mark.parametrize("geom", [(8, 2, 128, True, True), (6, 6, 64, True, False), (5, 1, 256, False, True),
                                   (16, 1, 64, True, True), (3, 3, 128, False, False)])
 @pytest.mark.parametrize("store", [True, False])
