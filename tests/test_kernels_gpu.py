@@ -766,6 +766,48 @@ def test_sampling_with_thousands_of_equal_logits_at_the_boundary(ops):
     _check_draws(ops, logits[1:2].repeat(3, 1), temps, torch.full((3,), 0.7), us, plain)
 
 
+def test_sampling_with_logits_that_are_not_numbers_and_small_vocabularies(ops):
+    """NaN counts as -inf, for the argmax and for a draw; a row that is -inf throughout gives
+    token 0 and one with +inf its first +inf; vocabularies smaller than a wave's group of
+    loads, and just beyond what the last scan takes, draw by the plain rule."""
+    from tests.plain import qwen3 as plain
+
+    nan, inf = float("nan"), float("inf")
+    for vocab in (3, 64, 1024, 1025, 5000):
+        gen = torch.Generator().manual_seed(vocab)
+        logits = 2.0 * torch.randn((6, vocab), generator=gen)
+        logits[0, ::2] = nan
+        logits[1, 1::3] = -inf
+        logits[2, :] = -inf
+        logits[3, :] = nan
+        logits[4, vocab // 2] = inf
+        logits[4, vocab - 1] = inf
+        cleaned = torch.where(torch.isnan(logits), torch.full_like(logits, -inf), logits)
+        want_top = [int(np.argmax(f64(cleaned)[r])) for r in range(6)]
+        want_top[2] = want_top[3] = 0
+        want_top[4] = vocab // 2
+        dev = logits.to(DEV)
+        assert ops.argmax(dev).cpu().tolist() == want_top, vocab
+        temps = torch.tensor([0.7, 1.0, 1.0, 0.5, 1.0, 0.0])
+        tops = torch.tensor([1.0, 0.8, 0.9, 1.0, 0.95, 0.9])
+        for trial in range(4):
+            us = torch.rand(6, generator=torch.Generator().manual_seed(trial))
+            got = ops.sample(dev, temps.to(DEV), tops.to(DEV), us.to(DEV)).cpu().tolist()
+            assert [got[2], got[3], got[4], got[5]] == [0, 0, vocab // 2, want_top[5]], (vocab, trial, got)
+            for r in (0, 1):
+                row = f64(cleaned)[r]
+                want = plain.sample_with_uniform(row, float(temps[r]), float(tops[r]), float(us[r]))
+                if got[r] != want:
+                    p = plain.sampling_distribution(row, float(temps[r]), float(tops[r]))
+                    cdf = np.cumsum(p)
+                    assert p[got[r]] > 0 and abs(cdf[min(got[r], want)] - float(us[r])) < 1e-5, (vocab, trial, r)
+    # a temperature so low that only the largest logit has mass: the argmax, whatever u
+    logits = 2.0 * torch.randn((3, 3000), generator=torch.Generator().manual_seed(1))
+    got = ops.sample(logits.to(DEV), torch.full((3,), 1e-3).to(DEV), torch.full((3,), 0.95).to(DEV),
+                     torch.tensor([0.0, 0.5, 0.999]).to(DEV)).cpu().tolist()
+    assert got == f64(logits).argmax(axis=1).tolist()
+
+
 def test_sampling_where_most_of_the_row_has_no_mass(ops):
     """Logits as a trained model's: a handful of tokens carry all the mass and whole stretches
     of the row lie too far below to have any, which the passes step over 256 tokens at a time.
