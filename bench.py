@@ -300,6 +300,9 @@ def main() -> int:
     parser.add_argument("--context-length", type=int, default=None,
                         help="longest request in tokens (default: the shape's max_position_embeddings)")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
+    parser.add_argument("--temperature", type=float, default=0.0,
+                        help="sample the timed run's tokens at this temperature (default 0: the largest logit)")
+    parser.add_argument("--top-p", type=float, default=1.0, help="with --temperature: the nucleus kept")
     parser.add_argument("--no-graphs", action="store_true", help="launch decode steps kernel by kernel")
     parser.add_argument("--no-points", action="store_true", help="skip the other batch sizes and contexts")
     parser.add_argument("--no-prefill", action="store_true")
@@ -339,7 +342,7 @@ def main() -> int:
         return 0
 
     serving = Serving(runner, cfg, args, args.batch, prompt_len, args.steps + args.warmup + (24 if args.mixed else 0),
-                      seed=1, room=1 if args.mixed else 0)
+                      seed=1, room=1 if args.mixed else 0, temperature=args.temperature, top_p=args.top_p)
     steps = min(args.steps, serving.ticks - args.warmup - (24 if args.mixed else 0))
     elapsed, mean_context = serving.timed_ticks(steps, args.warmup)
     mixed_ms = serving.mixed_tick_ms(repeats=5) if args.mixed else None
@@ -350,9 +353,10 @@ def main() -> int:
     achieved = step_bytes / (elapsed / steps)
 
     headline = (args.shape == "4b" and args.batch == 8 and prompt_len == PROMPT_LEN and args.dtype == "bfloat16"
-                and layers == shape["num_hidden_layers"])
+                and layers == shape["num_hidden_layers"] and args.temperature == 0)
+    drawn = f", temperature {args.temperature:g}, top-p {args.top_p:g}" if args.temperature > 0 else ""
     record = {
-        "metric": f"decode tokens/s, Qwen3-{args.shape.upper()} shape, batch {args.batch}, {prompt_len}-token prompts",
+        "metric": f"decode tokens/s, Qwen3-{args.shape.upper()} shape, batch {args.batch}, {prompt_len}-token prompts{drawn}",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": round(value / REFERENCE_DECODE_B8, 2) if headline else None, "dtype": dtype_key, "data": "synthetic",
