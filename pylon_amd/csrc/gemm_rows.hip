@@ -1,6 +1,7 @@
-// out[M, N] = x[M, K] * w[N, K]^T in bfloat16 for 17 to 64 rows of x: the matrix products of
-// a decode step with many requests, still bound by reading w once, but with x no longer
-// small beside a workgroup's share of w.
+// out[M, N] = x[M, K] * w[N, K]^T in bfloat16 for up to 64 rows of x a workgroup (up to 128 a
+// launch, as two halves with workgroups of their own): the matrix products of a decode step,
+// bound by reading w once, with x from 17 rows on no longer small beside a workgroup's share
+// of w.
 //
 // A workgroup of four wavefronts owns 64 or 128 columns of the output (each wave one or two
 // tiles of 16 rows of w) over a range of K; K is cut over blockIdx.y and every cut writes
@@ -81,7 +82,7 @@ template <int MT, int CT, bool GLU, int WAVES, typename TO>
 __device__ __forceinline__ void gemm_rows_body(
     TO* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int M, int N,
     int K, long long ldx, long long ldw, long long ldo, long long part_stride, int chunks_per_part,
-    int wg_cols) {
+    int wg_cols, int group) {
   typedef GrShape<MT, CT, WAVES> Shape;
   constexpr int QW = 4 / WAVES;  // quarters of every tile of x that a wave fills
   constexpr int STAGES = Shape::STAGES;
@@ -92,7 +93,7 @@ __device__ __forceinline__ void gemm_rows_body(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PYLON_WAVE);
   const int r = lane & 15, g = lane >> 4;
   constexpr int WAVE_COLS = (GLU ? 1 : CT) * 16;  // columns of the output per wave
-  const int wg_row0 = blockIdx.x * wg_cols;  // first row of w the descriptor covers
+  const int wg_row0 = group * wg_cols;  // first row of w the descriptor covers
   const int wg_end = (N - wg_row0 < wg_cols) ? N : wg_row0 + wg_cols;
   const int n0 = wg_row0 + wave * WAVE_COLS;
   const int n_end = (wg_end - n0 < WAVE_COLS) ? wg_end : n0 + WAVE_COLS;  // <= n0: a wave without columns
@@ -255,8 +256,23 @@ template <int MT, int CT, bool GLU, int WAVES, typename TO>
 __global__ __launch_bounds__(WAVES* PYLON_WAVE) void gemm_rows_kernel(
     TO* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, int M, int N,
     int K, long long ldx, long long ldw, long long ldo, long long part_stride, int chunks_per_part,
-    int wg_cols) {
-  gemm_rows_body<MT, CT, GLU, WAVES, TO>(out, x, w, M, N, K, ldx, ldw, ldo, part_stride, chunks_per_part, wg_cols);
+    int wg_cols, int groups, int row_split) {
+  // More than 64 rows of x go as two halves of `row_split` rows, each to workgroups of its
+  // own that take the same columns: blockIdx.x counts eight groups of columns for the first
+  // half, the same eight for the second, then the next eight, so that the two workgroups that
+  // stream the same rows of w start together and on the same die (a die takes every eighth
+  // workgroup), where the second finds in the cache what the first brought.
+  int group = blockIdx.x;
+  if (row_split > 0) {
+    const int half = (blockIdx.x >> 3) & 1;
+    group = ((blockIdx.x >> 4) << 3) | (blockIdx.x & 7);
+    if (group >= groups) return;  // the grid is padded to whole sixteens
+    x += static_cast<size_t>(half) * row_split * ldx;
+    out += static_cast<size_t>(half) * row_split * ldo;
+    M = (M - half * row_split < row_split) ? M - half * row_split : row_split;
+  }
+  gemm_rows_body<MT, CT, GLU, WAVES, TO>(out, x, w, M, N, K, ldx, ldw, ldo, part_stride, chunks_per_part, wg_cols,
+                                         group);
 }
 
 // How a product is laid over the chip: wavefronts per workgroup, workgroups along the columns,
@@ -297,29 +313,31 @@ static GrLaunch gr_launch_shape(int M, int N, int parts, int col_tiles, int glu,
 template <int MT, int CT, bool GLU, int WAVES>
 static void launch_rows_waves(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                               long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
-                              const GrLaunch& shape, hipStream_t stream) {
+                              const GrLaunch& shape, int row_split, hipStream_t stream) {
   const int chunks = (K + GR_CHUNK - 1) / GR_CHUNK;
   const int per_part = (chunks + parts - 1) / parts;
-  dim3 grid(shape.groups, parts), block(WAVES * PYLON_WAVE);
+  dim3 grid(row_split > 0 ? 2 * ((shape.groups + 7) / 8 * 8) : shape.groups, parts), block(WAVES * PYLON_WAVE);
   if (out_dtype == PYLON_F32)
     hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, GLU, WAVES, float>), grid, block, 0, stream, (float*)out,
                        (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part,
-                       shape.wg_cols);
+                       shape.wg_cols, shape.groups, row_split);
   else
     hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, GLU, WAVES, bf16_t>), grid, block, 0, stream, (bf16_t*)out,
                        (const uint16_t*)x, (const uint16_t*)w, M, N, K, ldx, ldw, ldo, part_stride, per_part,
-                       shape.wg_cols);
+                       shape.wg_cols, shape.groups, row_split);
 }
 
 // Workgroups of four waves, or of two where four would leave compute units without one.
 template <int MT, int CT, bool GLU>
 static void launch_rows(void* out, int out_dtype, const void* x, const void* w, int M, int N, int K,
                         long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
-                        const GrLaunch& shape, hipStream_t stream) {
+                        const GrLaunch& shape, int row_split, hipStream_t stream) {
   if (shape.waves == 2)
-    launch_rows_waves<MT, CT, GLU, 2>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, stream);
+    launch_rows_waves<MT, CT, GLU, 2>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape,
+                                      row_split, stream);
   else
-    launch_rows_waves<MT, CT, GLU, 4>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, stream);
+    launch_rows_waves<MT, CT, GLU, 4>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape,
+                                      row_split, stream);
 }
 
 // What pylon_gemm_rows would launch for these arguments on a device of `units` compute units
@@ -333,12 +351,14 @@ extern "C" int pylon_gemm_rows_shape(int M, int N, int parts, int col_tiles, int
   PYLON_REQUIRE(waves == 0 || waves == 2 || waves == 4, "gemm_rows_shape: waves is 0, 2 or 4");
   if (units <= 0) units = pylon_compute_units();
   PYLON_REQUIRE(units > 0, "gemm_rows_shape: no device to take the number of compute units from");
-  const GrLaunch l = gr_launch_shape(M, N, parts, col_tiles, glu, waves, units, cols);
+  // beyond 64 rows each half of the rows has workgroups of its own: shape[1] of them per half
+  const GrLaunch l = gr_launch_shape(M > 64 ? (M + 1) / 2 : M, N, parts, col_tiles, glu, waves, units, cols);
   shape[0] = l.waves, shape[1] = l.groups, shape[2] = l.wg_cols;
   return 0;
 }
 
-// x: [M, ldx] bf16, 1 <= M <= 64; w: [N, ldw] bf16 (with glu: [2N, ldw], gate rows first, then
+// x: [M, ldx] bf16, 1 <= M <= 128 (beyond 64 rows two halves of (M + 1) / 2 and the rest, each to
+// workgroups of its own); w: [N, ldw] bf16 (with glu: [2N, ldw], gate rows first, then
 // up rows); out: `parts` results [M, ldo] spaced part_stride elements apart (parts > 1 needs
 // float out and no glu).  col_tiles: tiles of 16 columns per wave, 1 or 2; with glu a wave
 // takes 16 gate rows and their 16 up rows.  waves: wavefronts per workgroup, 4 or 2 (0: two if
@@ -349,7 +369,7 @@ extern "C" int pylon_gemm_rows(void* out, int out_dtype, const void* x, const vo
                                long long ldx, long long ldw, long long ldo, int parts, long long part_stride,
                                int col_tiles, int glu, int waves, int cols, hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(out_dtype), "gemm_rows: unknown output dtype");
-  PYLON_REQUIRE(M >= 0 && M <= 64, "gemm_rows: takes at most 64 rows, got %d", M);
+  PYLON_REQUIRE(M >= 0 && M <= 128, "gemm_rows: takes at most 128 rows, got %d", M);
   PYLON_REQUIRE(N > 0 && K > 0, "gemm_rows: bad sizes N=%d K=%d", N, K);
   PYLON_REQUIRE(K % 8 == 0, "gemm_rows: K=%d must be a multiple of 8", K);
   PYLON_REQUIRE(ldx % 8 == 0 && ldw % 8 == 0, "gemm_rows: row strides must be multiples of 8 elements");
@@ -371,16 +391,19 @@ extern "C" int pylon_gemm_rows(void* out, int out_dtype, const void* x, const vo
   if (M == 0) return 0;
   const int units = pylon_compute_units();
   PYLON_REQUIRE(units > 0, "gemm_rows: the device's number of compute units is unknown");
-  const GrLaunch shape = gr_launch_shape(M, N, parts, col_tiles, glu, waves, units, cols);
+  // beyond 64 rows: two halves, each to workgroups of its own
+  const int row_split = M > 64 ? (M + 1) / 2 : 0;
+  const int rows_each = row_split > 0 ? row_split : M;
+  const GrLaunch shape = gr_launch_shape(rows_each, N, parts, col_tiles, glu, waves, units, cols);
   PYLON_REQUIRE(cols >= 0 && cols <= shape.waves * (glu ? 1 : col_tiles) * 16,
                 "gemm_rows: %d columns per workgroup are more than the tiles of its %d waves hold", cols, shape.waves);
 #define GO(MT)                                                                                              \
   do {                                                                                                      \
-    if (glu) launch_rows<MT, 2, true>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, stream); \
-    else if (col_tiles == 2) launch_rows<MT, 2, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, stream); \
-    else launch_rows<MT, 1, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, stream); \
+    if (glu) launch_rows<MT, 2, true>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, row_split, stream); \
+    else if (col_tiles == 2) launch_rows<MT, 2, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, row_split, stream); \
+    else launch_rows<MT, 1, false>(out, out_dtype, x, w, M, N, K, ldx, ldw, ldo, parts, part_stride, shape, row_split, stream); \
   } while (0)
-  switch ((M + 15) / 16) {
+  switch ((rows_each + 15) / 16) {
     case 1: GO(1); break;
     case 2: GO(2); break;
     case 3: GO(3); break;

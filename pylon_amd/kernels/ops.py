@@ -473,7 +473,8 @@ def gemm_tiled(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[tor
 
 
 SKINNY_ROWS = plan.FEW_ROWS    # one tile of rows of x
-STREAM_ROWS = plan.STREAM_ROWS  # most rows of x one launch of a weight-streaming kernel takes
+STREAM_ROWS = plan.STREAM_ROWS  # most rows of x a workgroup of a weight-streaming kernel takes
+SPLIT_ROWS = plan.SPLIT_ROWS    # most rows the rows kernel takes, as two halves
 
 
 def _streaming_ok(x: torch.Tensor, weight: torch.Tensor, rows: int) -> bool:
@@ -519,9 +520,10 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype
 def gemm_rows(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype = torch.bfloat16,
               parts: int = 1, col_tiles: int = 1, glu: bool = False, waves: int = 0, cols: int = 0,
               out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``x @ weight.T`` for at most 64 rows of bfloat16 ``x``: the rows of ``x`` pass through
+    """``x @ weight.T`` for at most 128 rows of bfloat16 ``x``: the rows of ``x`` pass through
     LDS once per workgroup of up to 64 (``col_tiles=1``) or 128 (``col_tiles=2``) columns and
-    ``weight`` is streamed once.  ``parts > 1`` cuts K into that many ranges and returns
+    ``weight`` is streamed once (beyond 64 rows each half of the rows has workgroups of its
+    own, and two that take the same columns run side by side).  ``parts > 1`` cuts K into that many ranges and returns
     float32 partial results ``[parts, M, N]`` for the consumer to add.  ``glu``: ``weight`` is
     a fused ``[2N, K]`` gate/up matrix and the result is ``silu(x @ gate.T) * (x @ up.T)``,
     rounded once.  ``waves``: wavefronts per workgroup, 4 or 2 (0: the kernel's choice);
@@ -593,9 +595,9 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: Optional[torch.d
 def linear_summed_later(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:
     """``x @ weight.T`` for a consumer that takes either the product in ``out_dtype`` or float32
     partial sums ``[parts, M, N]`` of it, to be added in order and rounded to ``out_dtype`` once
-    (:func:`attention_decode_fused` does): from 17 to 64 bfloat16 rows the weight-streaming
+    (:func:`attention_decode_fused` does): up to 128 bfloat16 rows the weight-streaming
     kernel with K cut over workgroups (:func:`plan.plan_summed_later`), else :func:`linear`."""
-    if out_dtype == torch.bfloat16 and _streaming_ok(x, weight, STREAM_ROWS):
+    if out_dtype == torch.bfloat16 and _streaming_ok(x, weight, SPLIT_ROWS):
         choice = plan.plan_summed_later(x.shape[0], *weight.shape, units=_lib.compute_units())
         if choice.kernel == "rows" and choice.parts > 1:
             return gemm_rows(x, weight, out_dtype=torch.float32, parts=choice.parts, col_tiles=choice.col_tiles)
@@ -604,12 +606,12 @@ def linear_summed_later(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: tor
 
 def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:
     """A product whose result is about to be added to the float32 residual stream.  For up
-    to 64 bfloat16 rows it comes back as unrounded float32 sums, which the fused residual norm
+    to 128 bfloat16 rows it comes back as unrounded float32 sums, which the fused residual norm
     adds: partial sums ``[parts, M, N]`` of a streaming kernel (K cut over workgroups), or,
-    for 17 to 64 rows of a matrix at which the library is faster, the library's float32
+    from 17 rows on for a matrix at which the library is faster, the library's float32
     result (:func:`plan.plan_residual`).  For more rows (prompt portions) it is the library's
     product rounded once to bfloat16."""
-    if _streaming_ok(x, weight, STREAM_ROWS):
+    if _streaming_ok(x, weight, SPLIT_ROWS):
         choice = plan.plan_residual(x.shape[0], *weight.shape, units=_lib.compute_units())
         if choice.kernel == "rows":
             return gemm_rows(x, weight, out_dtype=torch.float32, parts=choice.parts, col_tiles=choice.col_tiles)

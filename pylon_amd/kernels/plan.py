@@ -16,7 +16,8 @@ from __future__ import annotations
 from dataclasses import dataclass
 
 FEW_ROWS = 16      # one tile of rows of x
-STREAM_ROWS = 64   # most rows of x a weight-streaming kernel takes
+STREAM_ROWS = 64   # most rows of x a workgroup of a weight-streaming kernel takes
+SPLIT_ROWS = 128   # most rows the rows kernel takes as two halves, each to workgroups of its own
 TALL = 32768       # a matrix of at least this many rows (a vocabulary head) is "tall"
 UNITS = 256        # compute units of an MI355X; callers on a device pass its own count
 
@@ -81,7 +82,11 @@ def plan_residual(rows: int, n: int, k: int, units: int = UNITS) -> Product:
     14.3 us, 2560x9728 16.0 against 28.0, 4096x4096 11.0 against 15.1, 4096x12288 26.5 against
     37.5, 5120x5120 16.3 against 21.8, 5120x8192 22.9 against 28.9, 5120x17408 42 against 86,
     6144x6144 21.5 against 26.8, 10240x10240 48 against 60), except for wide matrices whose rows
-    are of a power-of-two length (8192x8192 36.4 against 33.7, 16384x4096 37.4 against 34.5)."""
+    are of a power-of-two length (8192x8192 36.4 against 33.7, 16384x4096 37.4 against 34.5).
+    From 65 to 128 rows the rows kernel takes the rows as two halves, each to workgroups of its
+    own, two that stream the same rows of w side by side on one die: 2560x9728 at 65, 96 and 128
+    rows 22.6, 23.0 and 26.2 us against the library's 26.2, 26.9 and 52.9 (bfloat16 result),
+    2560x4096 14.1, 14.3 and 16.8 against 20.9, 20.9 and 22.9; the same choices as for 64 rows."""
     few = rows <= FEW_ROWS
     if few:
         if deep_or_narrow(n, k) or n <= 8192:
@@ -108,6 +113,8 @@ def plan_projection(rows: int, n: int, k: int) -> Product:
     x of a workgroup that covers 64 of many columns weigh most here; a consumer that adds
     partial sums gets them (:func:`plan_summed_later`)."""
     few = rows <= FEW_ROWS
+    if rows > STREAM_ROWS:
+        return Product("library")
     if n >= TALL:
         if aliased_rows(k):
             return Product("rows", 1, 1) if rows <= 32 else Product("library")
@@ -128,14 +135,15 @@ def plan_summed_later(rows: int, n: int, k: int, units: int = UNITS) -> Product:
     From 17 to 64 rows the rows kernel so cut beats the library, which does not cut K: 6144 x
     2560 at 17, 32, 48 and 64 rows 9.0, 9.5, 10.8 and 11.7 us (four parts of 128 columns) against
     11.0, 11.8, 15.3 and 15.5; 6144 x 4096 11.8 to 14.9 against 14.5 to 17.9; 10240 x 5120 (two
-    parts) 21.5 to 28.1 against 24.4 to 32.8.  Without a cut as :func:`plan_projection`."""
+    parts) 21.5 to 28.1 against 24.4 to 32.8.  From 65 to 128 rows, as two halves: 6144 x 2560 15.4 to
+    18.2 us against the library's 20.9 to 21.3.  Without a cut as :func:`plan_projection`."""
     if n < TALL and rows <= FEW_ROWS:
         groups, parts = -(-n // 64), 1
         while parts < 4 and 2 * parts * groups <= units and k // (2 * parts) >= 256:
             parts *= 2
         if parts > 1:
             return Product("rows", parts, 1)
-    elif n < TALL and rows <= STREAM_ROWS:
+    elif n < TALL and rows <= SPLIT_ROWS:
         parts, col_tiles = rows_split(n, k, rows, units)
         if parts > 1:
             return Product("rows", parts, col_tiles)
@@ -155,6 +163,8 @@ def plan_gated(rows: int, n_half: int, k: int, row_stride: int) -> Product:
     13.8 to 14.3 (2x6144 x 2048 at 64 rows alone loses, 20.9 against 19.8).  A workgroup of the
     rows kernel sees its gate rows and, ``n_half`` rows further, its up rows through one
     descriptor, which spans at most 2 GB."""
+    if rows > STREAM_ROWS:  # 2x9728 x 2560 at 65 to 128 rows: 41 to 48 us against the library's 36 to 38
+        return Product("library")
     few = rows <= FEW_ROWS
     fits = (n_half + 64) * row_stride * 2 < 2 ** 31
     if fits and (not few or (not aliased_rows(k) and n_half >= 4096)):

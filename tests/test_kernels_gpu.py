@@ -240,13 +240,14 @@ def test_gemm_skinny(ops, shape):
 
 
 def test_gemm_rows_at_random_shapes(ops):
-    """Sixty seeded draws of every argument (rows 1 to 64, 1 to 700 columns, depths that are
-    multiples of 8 up to 1,496, parts beyond the number of chunks, both widths and wave
-    counts, the gated form) against a float64 product; and with any number of columns per
-    workgroup, down to one, the bits of the kernel's own choice."""
+    """Ninety seeded draws of every argument (rows 1 to 128, beyond 64 as two halves with
+    workgroups of their own; 1 to 700 columns, depths that are multiples of 8 up to 1,496,
+    parts beyond the number of chunks, both widths and wave counts, the gated form) against a
+    float64 product; and with any number of columns per workgroup, down to one, the bits of
+    the kernel's own choice."""
     rng = np.random.default_rng(2024)
-    for case in range(60):
-        m = int(rng.integers(1, 65))
+    for case in range(90):
+        m = int(rng.integers(1, 65)) if case < 60 else int(rng.integers(65, 129))
         k = 8 * int(rng.integers(1, 188))
         glu = bool(rng.integers(0, 2))
         n = int(rng.integers(1, 351)) * (2 if glu else 1) if glu else int(rng.integers(1, 701))
@@ -295,8 +296,14 @@ def test_gemm_rows(ops, shape):
     full = ops.gemm_rows(a.to(DEV), w.to(DEV), parts=4)
     alone = ops.gemm_rows(a[m // 2: m // 2 + 1].contiguous().to(DEV), w.to(DEV), parts=4)
     assert torch.equal(alone[:, 0], full[:, m // 2])
-    with pytest.raises(Exception, match="at most 64 rows"):
-        ops.gemm_rows(rnd((65, k), 34, torch.bfloat16).to(DEV), w.to(DEV))
+    with pytest.raises(Exception, match="at most 128 rows"):
+        ops.gemm_rows(rnd((129, k), 34, torch.bfloat16).to(DEV), w.to(DEV))
+    # beyond 64 rows the rows go as two halves: the same bits for a row as in a launch of its own
+    tall = torch.cat([a, rnd((100 - m, k), 37, torch.bfloat16)]) if m < 100 else a
+    both = ops.gemm_rows(tall.to(DEV), w.to(DEV), parts=4)
+    assert both.shape == (4, tall.shape[0], n)
+    assert torch.equal(both[:, : m], full) and torch.equal(
+        both[:, 99], ops.gemm_rows(tall[99:100].contiguous().to(DEV), w.to(DEV), parts=4)[:, 0])
     # rows of x and w that are slices of wider tensors (strides beyond K)
     wide_x = rnd((m, k + 24), 35, torch.bfloat16).to(DEV)
     wide_w = rnd((n, k + 40), 36, torch.bfloat16, 0.1).to(DEV)

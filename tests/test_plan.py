@@ -107,6 +107,22 @@ def test_a_projection_whose_consumer_adds_partial_sums_is_cut_over_k():
         assert plan.plan_summed_later(rows, 6144, 256).parts == 1
 
 
+def test_from_65_to_128_rows_the_products_that_are_added_later_stay_with_the_rows_kernel():
+    """Two halves of the rows, each to workgroups of its own, with the choices of 64 rows: out,
+    down and the q/k/v whose partial sums the attention adds.  Gate/up, the head and a q/k/v
+    that must come whole go to the library, as does everything beyond 128 rows."""
+    for name in SIZES:
+        hidden, q, kv, inter = SIZES[name]
+        for rows in (65, 100, 128):
+            for n, k in ((hidden, q), (hidden, inter)):
+                assert plan.plan_residual(rows, n, k) == plan.plan_residual(64, n, k), (name, rows, n, k)
+            assert plan.plan_summed_later(rows, q + 2 * kv, hidden) == plan.plan_summed_later(64, q + 2 * kv, hidden)
+            assert plan.plan_projection(rows, q + 2 * kv, hidden).kernel == "library"
+            assert plan.plan_projection(rows, VOCAB, hidden).kernel == "library"
+            assert plan.plan_gated(rows, inter, hidden, hidden).kernel == "library"
+    assert plan.SPLIT_ROWS == 128 and plan.STREAM_ROWS == 64
+
+
 def test_decode_attention_cuts_the_keys_of_few_long_requests_over_workgroups():
     """`ops.decode_cuts` is a pure function of the shape: up to 512 keys one workgroup per
     (token, head), as up to 767; beyond, powers of two of cuts of at least 192 keys while the workgroups stay

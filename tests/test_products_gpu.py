@@ -12,7 +12,7 @@ launch gets the same share of the columns, a whole number of rounds over the 256
 units, unless that would make it re-read more rows of x than it streams rows of w):
 
 =========  ========================  =====================================  ===================
-product    1, 8, 16 rows             17, 48, 64 rows                        65, 130 rows
+product    1, 8, 16 rows             17, 48, 64 rows                        130 rows
 =========  ========================  =====================================  ===================
 4b qkv     rows CT1 2w 256x1 c24     library, bfloat16                      library, bfloat16
 4b out     rows CT1 4w 64x4 c40      rows CT1 4w 64x4 c40 at 17 rows,       library, bfloat16
@@ -37,6 +37,10 @@ In front of the decode attention that prepares its own operands q/k/v may also c
 partial sums (``ops.linear_summed_later``): up to 16 rows rows CT1 4w 128x2 c48 (4B, 8B; the
 32B shape as above), from 17 to 64 rows rows CT2 4w 64x4 c96 (4B, 8B) and 128x2 c80 (32B), else
 as above.
+
+65 and 128 rows: the rows of x go as two halves, each to workgroups of its own, with the choices
+of 64 rows, for out, down and the q/k/v that a consumer adds; gate/up, the head and a plain q/k/v
+go to the library as at 130 rows.
 """
 import ctypes
 import zlib
@@ -51,7 +55,7 @@ DEV = "cuda:0"
 VOCAB = 151936
 # (hidden, q width, key/value width, feed-forward width)
 SIZES = {"4b": (2560, 4096, 1024, 9728), "8b": (4096, 4096, 1024, 12288), "32b": (5120, 8192, 1024, 25600)}
-ROWS = (1, 8, 16, 17, 48, 64, 65, 130)
+ROWS = (1, 8, 16, 17, 48, 64, 65, 128, 130)
 
 # (kernel, parts, col_tiles, (waves, groups, columns per workgroup)) for few (<= 16) and many
 # (17..64) rows; a dict where the many differ among themselves
@@ -148,8 +152,11 @@ def test_a_product_at_its_real_size(ops, model, product):
         xr = x[:rows].contiguous()
         if product in ("out", "down"):
             got = ops.linear_for_residual(xr, w, out_dtype=torch.bfloat16)
-            if rows <= 64:  # float32 sums, never rounded: whole, or K cut into parts
+            if rows <= 128:  # float32 sums, never rounded: whole, or K cut into parts
                 assert got.dtype == torch.float32
+                if rows > 64:  # two halves of the rows, the choices of 64 rows
+                    many64 = many[64] if isinstance(many, dict) else many
+                    assert chosen(model, product, rows, units)[:3] == many64[:3], (model, product, rows)
                 got = got.sum(0, dtype=torch.float64) if got.dim() == 3 else got
             else:
                 assert got.dtype == torch.bfloat16
@@ -165,10 +172,13 @@ def test_a_product_at_its_real_size(ops, model, product):
             from pylon_amd.kernels import plan
 
             c = plan.plan_summed_later(rows, n, k, units=units)
-            if rows <= 64 and c.parts > 1:
+            if rows <= 128 and c.parts > 1:
                 expected = EXPECT_SUMMED[model][0 if rows <= 16 else 1]
-                assert (c.kernel, c.parts, c.col_tiles, launch_shape(rows, n, c.parts, c.col_tiles, 0)) == \
-                    expected, (model, rows)
+                if rows <= 64:
+                    assert (c.kernel, c.parts, c.col_tiles, launch_shape(rows, n, c.parts, c.col_tiles, 0)) == \
+                        expected, (model, rows)
+                else:  # two halves of the rows, the choices of 64 rows
+                    assert (c.kernel, c.parts, c.col_tiles) == expected[:3], (model, rows)
                 assert later.dtype == torch.float32 and later.shape == (c.parts, rows, n)
                 total = later.sum(0, dtype=torch.float64).cpu().numpy()
                 assert np.abs(total - want[:rows]).max() <= 2e-6 * np.abs(want[:rows]).max(), (model, rows)
