@@ -73,7 +73,7 @@ def deep_or_narrow(n: int, k: int) -> bool:
 
 def plan_residual(rows: int, n: int, k: int, units: int = UNITS) -> Product:
     """A product about to be added to the float32 residual stream (out and down projections),
-    ``rows`` <= 64: float32 sums, never rounded, from whichever kernel.
+    ``rows`` <= 128: float32 sums, never rounded, from whichever kernel.
 
     Up to 16 rows the rows kernel beats the skinny one for deep, narrow and moderately wide
     matrices (2560x4096 at 8 rows: 6.2 against 8.3 us, 2560x9728 11.5 against 13.8, 5120x8192
@@ -98,7 +98,7 @@ def plan_residual(rows: int, n: int, k: int, units: int = UNITS) -> Product:
 
 
 def plan_projection(rows: int, n: int, k: int) -> Product:
-    """Any other product of ``rows`` <= 64 (q/k/v; the vocabulary head).
+    """Any other product (q/k/v; the vocabulary head); beyond 64 rows the library's.
 
     A head (tall matrix): the rows kernel with 128 columns per workgroup (151936 x 2560: 137 us
     against the skinny kernel's 154 at 8 rows; 173 against the library's 186 at 64 rows, 150
@@ -151,8 +151,8 @@ def plan_summed_later(rows: int, n: int, k: int, units: int = UNITS) -> Product:
 
 
 def plan_gated(rows: int, n_half: int, k: int, row_stride: int) -> Product:
-    """``silu(x gate^T) * (x up^T)`` over a fused matrix of ``2 * n_half`` rows, ``rows`` <= 64;
-    "library" means its float32 result followed by the activation kernel.
+    """``silu(x gate^T) * (x up^T)`` over a fused matrix of ``2 * n_half`` rows; "library" means
+    its product followed by the activation kernel (up to 64 rows its float32 result).
 
     Against the skinny kernel at 8 rows: 2x9728 x 2560 20 against 25 us, 2x25600 x 5120 90
     against 105, 2x17408 x 5120 63 against 76, 2x6144 x 2048 13.8 against 15.2; but 2x12288 x
