@@ -56,7 +56,9 @@ def weight_bytes(spec, dtype: torch.dtype, param_dtypes: Optional[Mapping[str, t
         size = param.element_size()
         if param_dtypes and path in param_dtypes:
             size = torch.empty((), dtype=param_dtypes[path]).element_size()
-        total += param.numel() * size
+        # a matrix whose rows lie apart in memory takes what its strides span
+        elements = param.shape[0] * param.stride(0) if param.dim() == 2 and param.shape[0] else param.numel()
+        total += max(elements, param.numel()) * size
     return total
 
 

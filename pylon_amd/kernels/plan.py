@@ -39,6 +39,17 @@ def aliased_rows(k: int) -> bool:
     return k % 4096 == 0
 
 
+def gated_row_padding(k: int, element_size: int) -> int:
+    """Elements to leave unused behind every row of a fused gate/up matrix of 16-bit elements
+    whose rows are of a power-of-two length of 8 KB or more.  Of all the products only this one
+    gains from rows that are a little longer in memory than they are (2x12288 x 4096: the rows
+    kernel at 8 rows 43.0 -> 34.7 us, which then beats the skinny kernel's 37.4; at 64 rows 47.3 ->
+    39.3; the library at 2,048 rows 333 -> 298; with 128 elements instead of 64 the same), the
+    others stay within 1 % either way: a workgroup's gate rows and its up rows, 12288 rows
+    further, otherwise meet in the same few memory channels."""
+    return 64 if element_size == 2 and aliased_rows(k) else 0
+
+
 def rows_split(n: int, k: int, rows: int = STREAM_ROWS, units: int = UNITS) -> tuple:
     """(parts, col_tiles) of the rows kernel for a product into the residual stream.
     Workgroups of 128 columns for deep matrices (beyond 16 rows, where the rows of x weigh
@@ -156,7 +167,8 @@ def plan_gated(rows: int, n_half: int, k: int, row_stride: int) -> Product:
 
     Against the skinny kernel at 8 rows: 2x9728 x 2560 20 against 25 us, 2x25600 x 5120 90
     against 105, 2x17408 x 5120 63 against 76, 2x6144 x 2048 13.8 against 15.2; but 2x12288 x
-    4096 44 against 39 (aliased rows) and 2x3072 x 1024 7.4 against 6.1 (a small matrix).
+    4096 44 against 39 (aliased rows; with the rows :func:`gated_row_padding` apart in memory
+    34.7 against 37.4) and 2x3072 x 1024 7.4 against 6.1 (a small matrix).
     Against the library and the activation kernel from 17 to 64 rows: 2x9728 x 2560 21 to 27
     against 30 to 34, 2x12288 x 4096 45 to 48 against 48 to 53, 2x17408 x 5120 67 to 86 against
     78 to 93, 2x25600 x 5120 91 to 105 against 94 to 107, 2x3072 x 1024 9.3 to 12.8 against
@@ -167,6 +179,6 @@ def plan_gated(rows: int, n_half: int, k: int, row_stride: int) -> Product:
         return Product("library")
     few = rows <= FEW_ROWS
     fits = (n_half + 64) * row_stride * 2 < 2 ** 31
-    if fits and (not few or (not aliased_rows(k) and n_half >= 4096)):
+    if fits and (not few or (not aliased_rows(row_stride) and n_half >= 4096)):
         return Product("rows", 1, 2)
     return Product("skinny") if few else Product("library")

@@ -77,8 +77,16 @@ class Part:
         self.param_roles: Dict[str, str] = {}
         self.children: Dict[str, "Part"] = {}
 
-    def add_param(self, name: str, shape, dtype: torch.dtype, device, role: str = "matrix") -> None:
-        self.params[name] = torch.empty(tuple(shape), dtype=dtype, device=device)
+    def add_param(self, name: str, shape, dtype: torch.dtype, device, role: str = "matrix",
+                  row_padding: int = 0) -> None:
+        """``row_padding``: elements left unused behind every row of a matrix in memory; the
+        parameter is then the view of its rows without them, with a row stride of its own."""
+        shape = tuple(shape)
+        if row_padding and len(shape) == 2:
+            self.params[name] = torch.empty((shape[0], shape[1] + row_padding), dtype=dtype,
+                                            device=device)[:, : shape[1]]
+        else:
+            self.params[name] = torch.empty(shape, dtype=dtype, device=device)
         self.param_roles[name] = role
 
     def add_child(self, name: str, part: "Part") -> "Part":

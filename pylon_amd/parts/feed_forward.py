@@ -5,7 +5,7 @@ from __future__ import annotations
 import torch
 
 from ..config.specs import GatedFeedForwardSpec
-from ..kernels import ops
+from ..kernels import ops, plan
 from .base import Part
 from .registry import register_part
 
@@ -17,7 +17,9 @@ class GatedFeedForward(Part):
             raise ValueError(f"activation {spec.activation!r} is not supported (only 'silu')")
         self.spec = spec
         self.dtype = dtype
-        self.add_param("gate_up", (2 * spec.intermediate_size, spec.hidden_size), dtype, device)
+        element_size = torch.empty((), dtype=dtype).element_size()
+        self.add_param("gate_up", (2 * spec.intermediate_size, spec.hidden_size), dtype, device,
+                       row_padding=plan.gated_row_padding(spec.hidden_size, element_size))
         self.add_param("down", (spec.hidden_size, spec.intermediate_size), dtype, device)
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:

@@ -59,6 +59,37 @@ def test_feed_forward_part():
         build_part("feed_forward", GatedFeedForwardSpec(8, 8, activation="gelu"), dtype=torch.float32, device=DEV)
 
 
+def test_feed_forward_part_whose_gate_up_rows_lie_apart_in_memory():
+    """A width whose rows are 8 KB in bfloat16: the fused gate/up matrix keeps 64 unused elements
+    behind every row (its rows then do not meet in the same few memory channels), the parameter
+    is the view without them, a load fills it like any other, and every product kernel that
+    takes part at some row count reads it through its row stride."""
+    from pylon_amd.config.specs import GatedFeedForwardSpec
+    from pylon_amd.engine.runner import weight_bytes
+    from pylon_amd.parts import build_part
+
+    hidden, inter = 4096, 4608
+    ff = build_part("feed_forward", GatedFeedForwardSpec(hidden_size=hidden, intermediate_size=inter),
+                    dtype=torch.bfloat16, device=DEV)
+    gate_up = ff.params["gate_up"]
+    assert gate_up.shape == (2 * inter, hidden) and gate_up.stride() == (hidden + 64, 1)
+    assert ff.params["down"].is_contiguous()
+    exact = build_part("feed_forward", GatedFeedForwardSpec(hidden_size=hidden, intermediate_size=8),
+                       dtype=torch.float32, device=DEV)
+    assert exact.params["gate_up"].is_contiguous()  # the 32-bit path's rows are left as they are
+    gate, up = rnd((inter, hidden), 4, 0.02).to(torch.bfloat16), rnd((inter, hidden), 5, 0.02).to(torch.bfloat16)
+    down = rnd((hidden, inter), 6, 0.02).to(torch.bfloat16)
+    gate_up[:inter].copy_(gate)   # as the loader does: a row range of the view
+    gate_up[inter:].copy_(up)
+    ff.params["down"].copy_(down)
+    for rows in (3, 16, 40, 64, 100, 300):  # skinny or rows kernel, rows kernel, library
+        x = rnd((rows, hidden), 7 + rows).to(torch.bfloat16)
+        got = ff.forward(x.to(DEV), None)
+        got = got.sum(0) if got.dim() == 3 else got
+        want = plain.gated_feed_forward(f64(x), f64(gate), f64(up), f64(down))
+        assert np.abs(f64(got) - want).max() <= 2e-2 * np.abs(want).max(), rows
+
+
 def test_position_part_and_registry():
     from pylon_amd.config.specs import PositionSpec
     from pylon_amd.parts import build_part
