@@ -41,13 +41,17 @@ def aliased_rows(k: int) -> bool:
 
 def gated_row_padding(k: int, element_size: int) -> int:
     """Elements to leave unused behind every row of a fused gate/up matrix of 16-bit elements
-    whose rows are of a power-of-two length of 8 KB or more.  Of all the products only this one
-    gains from rows that are a little longer in memory than they are (2x12288 x 4096: the rows
-    kernel at 8 rows 43.0 -> 34.7 us, which then beats the skinny kernel's 37.4; at 64 rows 47.3 ->
-    39.3; the library at 2,048 rows 333 -> 298; with 128 elements instead of 64 the same), the
-    others stay within 1 % either way: a workgroup's gate rows and its up rows, 12288 rows
-    further, otherwise meet in the same few memory channels."""
-    return 64 if element_size == 2 and aliased_rows(k) else 0
+    (of rows of at least 1,024 of them).
+    A workgroup's gate rows and its up rows, half the matrix further, otherwise tend to meet in
+    the same memory channels, most of all where a row is a power-of-two length of 8 KB or more:
+    2x12288 x 4096: the rows kernel at 8 rows 43.0 -> 34.7 us (which then beats the skinny
+    kernel's 37.4), at 64 rows 47.3 -> 39.3.  At other widths the streaming kernels gain little
+    (2x9728 x 2560 at 8 rows 20.1 -> 19.5 us) and the library's product for prompt portions some
+    (2,048 rows of 2x9728 x 2560: 212 -> 187 us alone, 0.2 ms of a 19.8 ms step): a whole step
+    at the Qwen3-4B shape 2.526 -> 2.516 ms decoding and 19.81 -> 19.60 ms for 2,048 prompt tokens,
+    old and new in turn on one device, three times.  The other products are within 1 % either
+    way and stay as they are; 192 elements do no better than 64."""
+    return 64 if element_size == 2 and k >= 1024 else 0  # not worth doubling a toy's matrix
 
 
 def rows_split(n: int, k: int, rows: int = STREAM_ROWS, units: int = UNITS) -> tuple:

@@ -60,8 +60,8 @@ def test_feed_forward_part():
 
 
 def test_feed_forward_part_whose_gate_up_rows_lie_apart_in_memory():
-    """A width whose rows are 8 KB in bfloat16: the fused gate/up matrix keeps 64 unused elements
-    behind every row (its rows then do not meet in the same few memory channels), the parameter
+    """A bfloat16 model's fused gate/up matrix keeps 64 unused elements behind every row (its rows
+    then do not meet in the same few memory channels: here a width whose rows are 8 KB), the parameter
     is the view without them, a load fills it like any other, and every product kernel that
     takes part at some row count reads it through its row stride."""
     from pylon_amd.config.specs import GatedFeedForwardSpec

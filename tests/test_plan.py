@@ -69,12 +69,12 @@ def test_rows_of_a_power_of_two_length_and_small_matrices_keep_the_other_kernels
     assert plan.plan_residual(8, 16384, 8192).kernel == "skinny"
 
 
-def test_gate_up_rows_of_a_power_of_two_length_are_kept_apart_in_memory():
-    """64 unused elements behind every 8 KB row of 16-bit elements, none otherwise; with them the
-    rows kernel takes the 8B gate/up at few rows too."""
-    assert plan.gated_row_padding(4096, 2) == 64 and plan.gated_row_padding(8192, 2) == 64
-    assert plan.gated_row_padding(2560, 2) == 0 and plan.gated_row_padding(5120, 2) == 0
+def test_gate_up_rows_are_kept_apart_in_memory():
+    """64 unused elements behind every row of 16-bit elements, none in the 32-bit path; with them
+    the rows kernel takes the 8B gate/up (rows of 8 KB) at few rows too."""
+    assert plan.gated_row_padding(4096, 2) == 64 and plan.gated_row_padding(2560, 2) == 64
     assert plan.gated_row_padding(4096, 4) == 0  # the 32-bit path's matrices stay as they are
+    assert plan.gated_row_padding(96, 2) == 0    # nor is a toy's matrix doubled
     assert plan.plan_gated(8, 12288, 4096, 4096).kernel == "skinny"
     assert plan.plan_gated(8, 12288, 4096, 4096 + 64) == plan.Product("rows", 1, 2)
     assert plan.plan_gated(64, 12288, 4096, 4096 + 64) == plan.Product("rows", 1, 2)
