@@ -16,10 +16,14 @@ pytestmark = pytest.mark.gpu
 BOUND = {"float32": 2e-5, "bfloat16": 2e-2}
 
 
-# Two corners the draws may miss: a width that is a multiple of 2 only with the largest head size
+# Corners the draws may miss: a width that is a multiple of 2 only with the largest head size
 # and seven query heads to a key/value head; a width that is a multiple of 4 only with the
-# smallest head size and sixteen query heads to one key/value head.
+# smallest head size and sixteen query heads to one key/value head; a width from which on a
+# bfloat16 model keeps the rows of its gate/up matrix apart in memory.
 CORNERS = {
+    "wide": (dict(num_hidden_layers=1, hidden_size=1032, num_attention_heads=6, num_key_value_heads=3, head_dim=64,
+                  intermediate_size=2050, vocab_size=333, rope_theta=1e6, rms_norm_eps=1e-6,
+                  tie_word_embeddings=True, max_position_embeddings=512), 32, (7, 90, 150)),
     "narrow": (dict(num_hidden_layers=2, hidden_size=50, num_attention_heads=7, num_key_value_heads=1, head_dim=512,
                     intermediate_size=34, vocab_size=131, rope_theta=12345.0, rms_norm_eps=3e-5,
                     tie_word_embeddings=True, max_position_embeddings=512), 16, (3, 70, 210)),
