@@ -622,12 +622,12 @@ def linear_for_residual(x: torch.Tensor, weight: torch.Tensor, *, out_dtype: tor
 
 
 def linear_glu(x: torch.Tensor, gate_up: torch.Tensor, *, out_dtype: torch.dtype) -> torch.Tensor:
-    """``silu(x @ gate.T) * (x @ up.T)`` for a fused ``[2I, K]`` gate/up matrix.  Up to 64
+    """``silu(x @ gate.T) * (x @ up.T)`` for a fused ``[2I, K]`` gate/up matrix.  Up to 128
     bfloat16 rows: the activation works on the float32 sums and its result is rounded once
-    (in a streaming kernel's epilogue; or, where the library is faster, from its float32
-    result: :func:`plan.plan_gated`).  More rows (prompt portions): the library's product
-    rounded to bfloat16 first."""
-    if _streaming_ok(x, gate_up, STREAM_ROWS) and x.is_cuda and gate_up.shape[0] % 2 == 0:
+    (in a streaming kernel's epilogue; or, where the library is faster and beyond 64 rows,
+    from its float32 result: :func:`plan.plan_gated`).  More rows (prompt portions): the
+    library's product rounded to bfloat16 first."""
+    if _streaming_ok(x, gate_up, SPLIT_ROWS) and x.is_cuda and gate_up.shape[0] % 2 == 0:
         choice = plan.plan_gated(x.shape[0], gate_up.shape[0] // 2, gate_up.shape[1], gate_up.stride(0))
         if choice.kernel == "rows":
             return gemm_rows(x, gate_up, out_dtype=out_dtype, glu=True)
